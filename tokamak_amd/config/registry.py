@@ -37,7 +37,7 @@ class Architecture:
 _ARCHITECTURES: dict[str, Architecture] = {}
 _PARTS: dict[tuple[str, str], type] = {}
 
-PART_FAMILIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+PART_FAMILIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "scale")
 
 
 def register_architecture(arch: Architecture, *, replace: bool = False) -> None:
@@ -155,6 +155,16 @@ def read_eos_token_ids(folder: Path) -> tuple[int, ...]:
     return ()
 
 
+def architecture_name(raw: dict) -> str:
+    """The architecture a ``config.json`` names: the first of ``architectures`` (a list), or
+    ``architecture`` (one name)."""
+    names = raw.get("architectures") or []
+    if names:
+        return names[0]
+    name = raw.get("architecture")
+    return name if isinstance(name, str) and name else "<missing>"
+
+
 def load_model_description(folder: str | Path) -> tuple[Architecture, Any, ModelPlan]:
     """Read ``config.json`` in ``folder``; return (architecture, typed config, plan)."""
     folder = Path(folder)
@@ -162,8 +172,6 @@ def load_model_description(folder: str | Path) -> tuple[Architecture, Any, Model
     if not path.is_file():
         raise FileNotFoundError(f"no config.json under {folder}")
     raw = json.loads(path.read_text())
-    names = raw.get("architectures") or []
-    name = names[0] if names else "<missing>"
-    arch = get_architecture(name)
+    arch = get_architecture(architecture_name(raw))
     config = arch.parse(raw, read_eos_token_ids(folder))
     return arch, config, arch.plan(config)

@@ -579,8 +579,49 @@ TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, hipSt
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// out[n, c] = scale[c] * (wa * a[n, c] + wb * b[n, c]), float32: the sum of a layer's parallel
+// branches, each with its weight, times a per-coordinate layer scale.  a and b are each T,
+// float32, or float32 partial sums of a split product; b may be absent.
+template <typename T>
+__device__ __forceinline__ float branch_value(const void* p, int f32, int parts, long part_stride, size_t idx) {
+  if (!f32) return Elem<T>::load(reinterpret_cast<const T*>(p) + idx);
+  const float* f = reinterpret_cast<const float*>(p);
+  float s = f[idx];
+  for (int i = 1; i < parts; ++i) s += f[idx + (size_t)i * part_stride];
+  return s;
+}
+
+template <typename T>
+__global__ void scaled_sum_kernel(const void* __restrict__ a, int a_f32, int a_parts, long a_stride, float wa,
+                                  const void* __restrict__ b, int b_f32, int b_parts, long b_stride, float wb,
+                                  const float* __restrict__ scale, float* __restrict__ out, int H, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float v = wa * branch_value<T>(a, a_f32, a_parts, a_stride, idx);
+  if (b != nullptr) v = fmaf(wb, branch_value<T>(b, b_f32, b_parts, b_stride, idx), v);
+  if (scale != nullptr) v *= scale[idx % H];
+  out[idx] = v;
+}
+
+TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long a_stride, float wa,
+                         const void* b, int b_f32, int b_parts, long b_stride, float wb, const float* scale,
+                         float* out, int N, int H, hipStream_t stream) {
+  if (N <= 0 || H <= 0) return 0;
+  const size_t total = (size_t)N * H;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == 0)
+    scaled_sum_kernel<float><<<blocks, 256, 0, stream>>>(a, a_f32, a_parts, a_stride, wa, b, b_f32, b_parts,
+                                                         b_stride, wb, scale, out, H, total);
+  else
+    scaled_sum_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, a_f32, a_parts, a_stride, wa, b, b_f32, b_parts,
+                                                          b_stride, wb, scale, out, H, total);
+  return launch_status();
+}
+
 // the same entry points in slot form (slots.h), for launch lists
 TK_SLOTS(tk_add_rmsnorm)
 TK_SLOTS(tk_rope_tables)
 TK_SLOTS(tk_qknorm_rope_store)
 TK_SLOTS(tk_silu_mul)
+TK_SLOTS(tk_scaled_sum)

@@ -175,6 +175,24 @@ _SIGS = {
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
         "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "tk_scaled_sum": [c_int, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float,
+                          c_void_p, c_void_p, c_int, c_int, c_void_p],
+    },
+    "attention_pooled": {
+        "tk_bias_norm_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                               c_int, c_float, c_int, c_void_p],
+        "tk_pooled_window_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_float, c_void_p],
+    },
+    "recurrent": {
+        "tk_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                           c_int, c_int, c_void_p],
+        "tk_tanh": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_long, c_void_p],
+        "tk_wkv_scan": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p,
+                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
+                        c_void_p],
     },
     "gemm_tiled": {
         "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
@@ -431,6 +449,157 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _note(f"{n}x{two_i // 2}", n * two_i * out.element_size() * 1.5)
     _check(_fn("elementwise", "tk_silu_mul")(_code(out.dtype), _p(gate_up), _p(out), n, two_i // 2,
                                              _stream()), "silu_mul")
+
+
+def _branch(t: torch.Tensor | None, rows: int, width: int, dtype: torch.dtype, what: str):
+    """(pointer, is_f32, parts, part_stride) of a contiguous [rows, width] input in ``dtype`` or
+    float32, or of float32 partial sums [parts, rows, width]."""
+    if t is None:
+        return _p(None), 0, 1, 0
+    _need(t.is_contiguous() and t.shape[-2] == rows, f"{what} must be contiguous with {rows} rows")
+    is_f32, parts, stride = _partials(t, rows, width, dtype, what)
+    return _p(t), is_f32, parts, stride
+
+
+def scaled_sum(a: torch.Tensor, weight_a: float, b: torch.Tensor | None, weight_b: float,
+               scale: torch.Tensor | None, out: torch.Tensor, dtype: torch.dtype) -> None:
+    """out = scale * (weight_a * a + weight_b * b), float32 [N, H].  ``a`` and ``b`` are each
+    [N, H] in ``dtype`` or float32, or float32 partial sums [P, N, H]; ``b`` and ``scale`` [H]
+    may be None."""
+    _gpu(a, b, scale, out)
+    n, h = out.shape
+    _need(out.dtype == torch.float32, "the scaled sum is float32")
+    _need(scale is None or (scale.dtype == torch.float32 and scale.numel() == h), "the scale is float32 [H]")
+    pa, fa, na, sa = _branch(a, n, h, dtype, "a")
+    pb, fb, nb, sb = _branch(b, n, h, dtype, "b")
+    _note(f"{n}x{h}", n * h * (4 + a.element_size() * na + (0 if b is None else b.element_size() * nb)))
+    _check(_fn("elementwise", "tk_scaled_sum")(_code(dtype), pa, fa, na, sa, float(weight_a), pb, fb, nb, sb,
+                                               float(weight_b), _p(scale), _p(out), n, h, _stream()), "scaled_sum")
+
+
+def bias_norm_store(qkv: torch.Tensor, bias: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
+                    positions: torch.Tensor, req_of_token: torch.Tensor, tables: torch.Tensor, q_out: torch.Tensor,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor, *, q_width: int, k_width: int, v_width: int,
+                    page_size: int, eps: float, store: bool = True) -> None:
+    """q/k/v projection output plus ``bias``; q and k each divided by the root mean square of
+    their whole row and multiplied by ``q_weight`` / ``k_weight``; q to ``q_out`` [N, q_width], k
+    and v into the pages (``[page][token][width]``) of each token's request."""
+    _gpu(qkv, bias, q_weight, k_weight, positions, req_of_token, tables, q_out, k_cache, v_cache)
+    n = q_out.shape[0]
+    total = q_width + k_width + v_width if store else q_width
+    dtype = q_out.dtype
+    _need(q_out.shape == (n, q_width) and k_cache.dtype == dtype and v_cache.dtype == dtype, "q/k/v outputs disagree")
+    _need(bias.dtype == torch.float32 and bias.numel() == q_width + k_width + v_width, "one float32 bias per projected coordinate")
+    _need(q_weight.dtype == torch.float32 and q_weight.numel() == q_width and k_weight.dtype == torch.float32
+          and k_weight.numel() == k_width, "norm weights are float32 over the whole projection")
+    _need(positions.numel() >= n and req_of_token.numel() >= n and tables.dim() == 2 and tables.dtype == torch.int32,
+          "step descriptor arrays are too short")
+    _need(k_cache.dim() == 2 and k_cache.shape[1] == k_width * page_size and v_cache.shape[1] == v_width * page_size
+          and k_cache.shape[0] == v_cache.shape[0], "cache arrays do not have the page layout")
+    p, is_f32, parts, stride = _branch(qkv, n, total, dtype, "qkv")
+    _note(f"{n}x{total}", n * total * (qkv.element_size() * parts + dtype.itemsize))
+    _check(_fn("attention_pooled", "tk_bias_norm_store")(
+        _code(dtype), p, is_f32, parts, stride, _p(bias), _p(q_weight), _p(k_weight), _p(positions),
+        _p(req_of_token), _p(tables), tables.shape[1], _p(q_out), _p(k_cache), _p(v_cache), n, q_width, k_width,
+        v_width, page_size, float(eps), int(bool(store)), _stream()), "bias_norm_store")
+
+
+POOLED_LDS_BYTES = 144 * 1024      # of a CU's 160 KB
+POOLED_ACC = 16                    # outputs a thread of the attention kernel accumulates
+
+
+def pooled_window_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, longest_span: int) -> tuple[int, int, int]:
+    """(rows a block takes, entries a chunk, threads a block) for the pooled-window attention
+    kernel: up to 8 consecutive rows of a portion share the keys and values a block stages;
+    single tokens take a block each."""
+    threads = 256
+    while num_heads * vdim > POOLED_ACC * threads and threads < 1024:
+        threads *= 2
+    _need(num_heads * vdim <= POOLED_ACC * threads, f"{num_heads} heads of {vdim} values are more than the kernel accumulates")
+    rows = 1 if longest_span <= 1 else max(1, min(8, POOLED_ACC * threads // (num_heads * vdim)))
+    while True:
+        fixed = rows * num_heads * dim + 2 * rows * num_heads + num_heads * num_heads
+        per_entry = num_kv_heads * (dim + vdim) + 2 + 2 * rows * num_heads
+        chunk = min(64, (POOLED_LDS_BYTES // 4 - fixed) // per_entry)
+        if chunk >= 8 or rows == 1:
+            break
+        rows //= 2
+    _need(chunk >= 1, "the heads of this attention do not fit the kernel's LDS")
+    return rows, chunk, threads
+
+
+def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,
+                            batch, talk: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
+                            dim: int, vdim: int, window: int, pool: int, page_size: int, scale: float) -> None:
+    """Attention of every row of the step over its request's pages: the last ``window``
+    positions one by one, complete blocks of ``pool`` positions behind them by the means of
+    their keys and values, one softmax over both, the heads' weights mixed by ``talk`` [H, H]."""
+    _gpu(q, k_cache, v_cache, tables, talk, out)
+    n = q.shape[0]
+    dtype = q.dtype
+    _need(q.shape == (n, num_heads * dim) and out.shape == (n, num_heads * vdim) and out.dtype == dtype, "q/out shapes disagree")
+    _need(k_cache.dtype == dtype and v_cache.dtype == dtype and k_cache.shape[1] == num_kv_heads * dim * page_size
+          and v_cache.shape[1] == num_kv_heads * vdim * page_size, "cache arrays do not have the page layout")
+    _need(talk.dtype == torch.float32 and talk.shape == (num_heads, num_heads), "the head-mixing matrix is float32 [H, H]")
+    _need(num_heads % num_kv_heads == 0 and window >= 1 and pool >= 1, "bad attention sizes")
+    _need(batch.num_tokens == n and tables.shape[0] == batch.num_requests and tables.dtype == torch.int32,
+          "block tables do not match the step")
+    _need(-(-batch.max_seq_len // page_size) <= tables.shape[1], "a block table is shorter than its request")
+    rows, chunk, threads = pooled_window_plan(num_heads, num_kv_heads, dim, vdim, batch.max_q_len)
+    _note(f"{n}x{num_heads}x{dim}", 0.0, 0.0)
+    _check(_fn("attention_pooled", "tk_pooled_window_attention")(
+        _code(dtype), _p(q), _p(k_cache), _p(v_cache), _p(out), _p(batch.positions), _p(batch.req_of_token),
+        _p(batch.q_start), _p(tables), tables.shape[1], _p(talk), n, num_heads, num_kv_heads, dim, vdim, window, pool,
+        page_size, rows, chunk, threads, float(scale), _stream()), "pooled_window_attention")
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, last: torch.Tensor, out: torch.Tensor, batch) -> None:
+    """out[s, n] = h[n] + (h[n - 1] - h[n]) * mu[s]; the row before a request's first token of
+    the step is ``last[slot]`` (float32 [slots, W]), which then takes the request's last row."""
+    _gpu(h, mu, last, out)
+    n, w = h.shape
+    s = mu.shape[0]
+    _need(mu.dtype == torch.float32 and mu.shape == (s, w) and last.dtype == torch.float32 and last.shape[1] == w,
+          "mix weights and the kept row are float32 of the input's width")
+    _need(out.shape == (s, n, w) and out.dtype == h.dtype and batch.num_tokens == n, "token shift shapes disagree")
+    _note(f"{n}x{w}x{s}", n * w * h.element_size() * (1 + s))
+    _check(_fn("recurrent", "tk_token_shift")(_code(h.dtype), _p(h), _p(mu), _p(last), _p(out), _p(batch.req_of_token),
+                                               _p(batch.q_start), _p(batch.state_slots), n, w, s, _stream()), "token_shift")
+
+
+def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = tanh(x); ``x`` [N, W] in out's dtype or float32, or float32 partial sums [P, N, W]."""
+    _gpu(x, out)
+    n, w = out.shape
+    p, is_f32, parts, stride = _branch(x, n, w, out.dtype, "x")
+    _check(_fn("recurrent", "tk_tanh")(_code(out.dtype), p, is_f32, parts, stride, _p(out), n * w, _stream()), "tanh")
+
+
+WKV_MAX_DIM = 256
+
+
+def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, decay_in: torch.Tensor,
+             w0: torch.Tensor, u: torch.Tensor, gain: torch.Tensor, state: torch.Tensor, out: torch.Tensor, batch,
+             *, heads: int, dim: int, eps: float) -> None:
+    """Per request and head, over the step's tokens in order: o = (S + diag(u) k v^T)^T r, then
+    S <- diag(exp(-exp(decay_in + w0))) S + k v^T (S float32 [slots, heads, dim, dim], kept);
+    out = o / rms(o) * gain * silu(gate).  r, k, v, gate, out: [N, heads * dim]."""
+    _gpu(r, k, v, gate, decay_in, w0, u, gain, state, out)
+    n, hd = out.shape
+    dtype = out.dtype
+    _need(hd == heads * dim and 1 <= dim <= WKV_MAX_DIM, f"the scan takes heads of up to {WKV_MAX_DIM} channels")
+    for t in (r, k, v, gate):
+        _need(t.shape == (n, hd) and t.dtype == dtype, "scan operands are [N, heads * dim] in one dtype")
+    for t in (w0, u, gain):
+        _need(t.dtype == torch.float32 and t.numel() == hd, "decay offset, bonus and gain are float32 [heads * dim]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, dim), "the state is float32 [slots, heads, dim, dim]")
+    _need(batch.num_tokens == n, "the step's descriptor does not match")
+    p, is_f32, parts, stride = _branch(decay_in, n, hd, dtype, "decay_in")
+    _note(f"{n}x{heads}x{dim}", n * hd * 6 * r.element_size(), 4.0 * n * heads * dim * dim)
+    _check(_fn("recurrent", "tk_wkv_scan")(
+        _code(dtype), _p(r), _p(k), _p(v), _p(gate), p, is_f32, parts, stride, _p(w0), _p(u), _p(gain), _p(state),
+        _p(batch.q_start), _p(batch.state_slots), _p(out), batch.num_requests, heads, dim, float(eps), _stream()),
+        "wkv_scan")
 
 
 FEWROWS_MAX_ROWS = 64          # float32 products of up to this many rows stream the weights, a lane a weight row,

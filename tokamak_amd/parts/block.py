@@ -5,6 +5,7 @@ from __future__ import annotations
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels.linear import Added, StreamSink
 from tokamak_amd.parts.base import Block
+from tokamak_amd.parts.scale import scaled_sum
 
 
 class PreNormBlock(Block):
@@ -59,4 +60,50 @@ def _sink(producer, next_norm, resid) -> dict:
     return {"add_into": StreamSink(resid, None)}
 
 
+class ParallelMixersBlock(Block):
+    """x = x + scale_1 * (left_weight * left(norm(x)) + right_weight * right(norm(x)));
+    x = x + scale_2 * feed_forward(norm(x)).
+
+    Two mixers side by side read the same normed input, each with a cache slot of its own.
+    ``mixer_scale`` and ``feed_forward_scale`` are per-coordinate layer scales (absent: ones);
+    the feed-forward with its norm and scale may be absent altogether.  The weighted sum and
+    the layer scale are formed in float32 from the branches' products, and the norm that reads
+    the stream next adds the result into it.
+    """
+
+    roles = ("mixer_norm", "left", "right")
+    optional = ("mixer_scale", "feed_forward_norm", "feed_forward", "feed_forward_scale")
+    replays_parts = True
+
+    def __init__(self, parts, *, left_weight: float = 1.0, right_weight: float = 1.0) -> None:
+        super().__init__(parts)
+        self.left_weight, self.right_weight = float(left_weight), float(right_weight)
+        self.mixer_norm, self.left, self.right = parts["mixer_norm"], parts["left"], parts["right"]
+        self.mixer_scale = parts.get("mixer_scale")
+        self.feed_forward = parts.get("feed_forward")
+        self.feed_forward_norm = parts.get("feed_forward_norm")
+        self.feed_forward_scale = parts.get("feed_forward_scale")
+        if (self.feed_forward is None) != (self.feed_forward_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        if self.feed_forward is None and self.feed_forward_scale is not None:
+            raise ValueError("a feed-forward scale without a feed-forward")
+        self.entry_norm = self.mixer_norm
+
+    def forward(self, resid, pending, batch, store, writes_cache):
+        h = self.mixer_norm.forward(resid, pending)
+        left = self.left.forward(h, batch, store["left"], writes_cache, None)
+        right = self.right.forward(h, batch, store["right"], writes_cache, None)
+        dim, dtype = resid.shape[1], h.dtype
+        weight = None if self.mixer_scale is None else self.mixer_scale.weight
+        pending = scaled_sum(left, self.left_weight, right, self.right_weight, weight, dim, dtype)
+        if self.feed_forward is None:
+            return pending
+        h = self.feed_forward_norm.forward(resid, pending)
+        out = self.feed_forward.forward(h, batch)
+        if self.feed_forward_scale is None:
+            return out
+        return scaled_sum(out, 1.0, None, 0.0, self.feed_forward_scale.weight, dim, dtype)
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "parallel_mixers", ParallelMixersBlock)

@@ -17,16 +17,17 @@ class TokenEmbedding(Embedding):
 
     capturable = True
 
-    def __init__(self, *, vocab_size: int, dim: int, dtype, device) -> None:
+    def __init__(self, *, vocab_size: int, dim: int, dtype, device, tensor: str = "weight") -> None:
         super().__init__(dtype=dtype, device=device)
         self.vocab_size, self.dim = int(vocab_size), int(dim)
+        self.tensor = str(tensor)       # the matrix's name behind the part's prefix
         self.weight: torch.Tensor | None = None
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
-        return {prefix + "weight": TensorSpec((self.vocab_size, self.dim))}
+        return {prefix + self.tensor: TensorSpec((self.vocab_size, self.dim))}
 
     def bind(self, prefix: str, fetch: Fetch) -> None:
-        self.weight = fetch(prefix + "weight")
+        self.weight = fetch(prefix + self.tensor)
 
     def tied_matrix(self) -> torch.Tensor:
         return self.weight
@@ -43,19 +44,20 @@ class LinearHead(Head):
 
     capturable = True
 
-    def __init__(self, *, vocab_size: int, dim: int, tied: bool, dtype, device) -> None:
+    def __init__(self, *, vocab_size: int, dim: int, tied: bool, dtype, device, tensor: str = "weight") -> None:
         super().__init__(dtype=dtype, device=device)
         self.vocab_size, self.dim, self.tied = int(vocab_size), int(dim), bool(tied)
+        self.tensor = str(tensor)
         self.weight: torch.Tensor | None = None
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         # a tied checkpoint may still carry its own copy: it is skipped
         # (reference: src/tokamak/model/loader.py:79-80)
-        return {prefix + "weight": TensorSpec((self.vocab_size, self.dim), ignored=self.tied)}
+        return {prefix + self.tensor: TensorSpec((self.vocab_size, self.dim), ignored=self.tied)}
 
     def bind(self, prefix: str, fetch: Fetch) -> None:
         if not self.tied:
-            self.weight = fetch(prefix + "weight")
+            self.weight = fetch(prefix + self.tensor)
 
     def tie(self, embedding: Embedding) -> None:
         weight = embedding.tied_matrix()

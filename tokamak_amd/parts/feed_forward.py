@@ -22,24 +22,24 @@ class SwiGLU(FeedForward):
     fuses_residual = True
     replayable = True
 
-    def __init__(self, *, hidden_size: int, intermediate_size: int, dtype, device) -> None:
+    def __init__(self, *, hidden_size: int, intermediate_size: int, dtype, device,
+                 names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
         super().__init__(dtype=dtype, device=device)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.names = tuple(names)       # gate, up, down behind the part's prefix
         self.gate_up: torch.Tensor | None = None
         self.down: torch.Tensor | None = None
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         h, i = self.hidden_size, self.intermediate_size
-        return {
-            prefix + "gate_proj.weight": TensorSpec((i, h)),
-            prefix + "up_proj.weight": TensorSpec((i, h)),
-            prefix + "down_proj.weight": TensorSpec((h, i)),
-        }
+        gate, up, down = self.names
+        return {prefix + gate: TensorSpec((i, h)), prefix + up: TensorSpec((i, h)), prefix + down: TensorSpec((h, i))}
 
     def bind(self, prefix: str, fetch: Fetch) -> None:
-        self.gate_up = torch.cat([fetch(prefix + "gate_proj.weight"), fetch(prefix + "up_proj.weight")], dim=0).contiguous()
-        self.down = fetch(prefix + "down_proj.weight")
+        gate, up, down = self.names
+        self.gate_up = torch.cat([fetch(prefix + gate), fetch(prefix + up)], dim=0).contiguous()
+        self.down = fetch(prefix + down)
 
     def forward(self, h, batch, add_into=None):
         return linear(gated_linear(h, self.gate_up), self.down, allow_partials=True, add_into=add_into)

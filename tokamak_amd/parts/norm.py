@@ -23,17 +23,18 @@ class RMSNorm(Norm):
     fuses_residual = True
     replayable = True
 
-    def __init__(self, *, dim: int, eps: float, dtype, device) -> None:
+    def __init__(self, *, dim: int, eps: float, dtype, device, tensor: str = "weight") -> None:
         super().__init__(dtype=dtype, device=device)
         self.dim = int(dim)
         self.eps = float(eps)
+        self.tensor = str(tensor)       # the weight's name behind the part's prefix
         self.weight: torch.Tensor | None = None
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
-        return {prefix + "weight": TensorSpec((self.dim,), role="vector")}
+        return {prefix + self.tensor: TensorSpec((self.dim,), role="vector")}
 
     def bind(self, prefix: str, fetch: Fetch) -> None:
-        self.weight = fetch(prefix + "weight")
+        self.weight = fetch(prefix + self.tensor)
 
     def sink(self, resid: torch.Tensor) -> StreamSink:
         return StreamSink(resid, self.weight)
@@ -51,4 +52,17 @@ class RMSNorm(Norm):
         return out
 
 
+class ScalarRMSNorm(RMSNorm):
+    """RMSNorm whose gain is a single number for all coordinates:
+    out = x * rsqrt(mean(x^2) + eps) * g.  The checkpoint holds g as a tensor without
+    dimensions; it is spread over the row once, at binding, and the kernels of ``RMSNorm`` run."""
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        return {prefix + self.tensor: TensorSpec((), role="vector")}
+
+    def bind(self, prefix: str, fetch: Fetch) -> None:
+        self.weight = fetch(prefix + self.tensor).reshape(1).expand(self.dim).contiguous()
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "scalar_rmsnorm", ScalarRMSNorm)

@@ -39,7 +39,7 @@ def validate(expected: Mapping[str, TensorSpec], found: Mapping[str, tuple]) -> 
     mismatched = [
         (n, found[n][0], s.shape)
         for n, s in expected.items()
-        if n in found and not s.ignored and tuple(found[n][0]) != tuple(s.shape)
+        if n in found and not s.ignored and not s.fits(found[n][0])
     ]
     if missing or unexpected or mismatched:
         raise WeightError(missing, unexpected, mismatched)

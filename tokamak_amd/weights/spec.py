@@ -18,10 +18,13 @@ class TensorSpec:
     float32, tables as int32.  A matrix that must not be rounded (a router, a decay
     table) says ``held="float32"`` and stays a matrix.
 
+    A dimension given as None is free: the checkpoint's tensor fixes it (a low rank that no
+    configuration key names), and the part reads it off the tensor it is given.
+
     ``optional`` tensors may be absent; ``ignored`` ones may be present and are
     skipped (a tied head's own copy of the embedding)."""
 
-    shape: tuple[int, ...]
+    shape: tuple[int | None, ...]
     role: str = "matrix"
     optional: bool = False
     ignored: bool = False
@@ -32,6 +35,10 @@ class TensorSpec:
             raise ValueError(f"role must be matrix, vector or table, got {self.role!r}")
         if self.held not in (None, "compute", "float32", "int32", "stored"):
             raise ValueError(f"held must be compute, float32, int32 or stored, got {self.held!r}")
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(want is None or want == got for want, got in zip(self.shape, shape))
 
     @property
     def holding(self) -> str:
