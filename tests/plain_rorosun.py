@@ -10,7 +10,6 @@ Weights are a dict name -> tensor with the checkpoint's names.
 from __future__ import annotations
 
 import json
-import math
 from pathlib import Path
 
 import torch
@@ -26,10 +25,6 @@ def rms(x: torch.Tensor, eps: float) -> torch.Tensor:
 def scalar_norm(x, g, eps):
     """RMS norm whose gain is one number for all coordinates."""
     return rms(x, eps) * g
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def silu(z):
