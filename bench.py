@@ -577,63 +577,20 @@ def run_latency(args) -> int:
     return 0
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256, help="timed decode steps of a pass (the headline workload: 256)")
-    ap.add_argument("--warmup", type=int, default=8, help="untimed decode steps before the timed passes")
-    ap.add_argument("--repeats", type=int, default=3, help="timed passes; the median is reported")
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--prompt", type=int, default=2048, help="prompt tokens of every request")
-    ap.add_argument("--context", type=int, default=None,
-                    help="instead of --prompt: the timed steps end when each request holds this many tokens")
-    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
-    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
-    ap.add_argument("--no-peaks", action="store_true", help="skip the microbenchmarks of this GPU's peaks")
-    ap.add_argument("--no-tune", action="store_true",
-                    help="take the library's first algorithm for long portions' products instead of timing its candidates")
-    ap.add_argument("--profile", action="store_true", help="add per-kernel times of one decode and one prefill step")
-    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
-                    help="run only one part (for an external profiler); the other part's figures are null")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace", "attention", "latency"],
-                    help="decode: the headline measurement; continuous: LLM.generate over many requests; "
-                         "trace: the reference's 32-request throughput trace at 1, 4 and 16 running requests; "
-                         "attention: the reference's decode-attention microbenchmark; "
-                         "latency: its single-sequence latency measurement (512 + 128 tokens)")
-    ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
-    ap.add_argument("--shape", default="qwen3-8b",
-                    help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
-    ap.add_argument("--requests", type=int, default=256)
-    ap.add_argument("--max-batch", type=int, default=64)
-    ap.add_argument("--prompt-tokens", default="32,1024", help="continuous workload: MIN,MAX prompt length")
-    ap.add_argument("--output-tokens", default="16,256", help="continuous workload: MIN,MAX output length")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
-        return 2
-    if args.workload == "continuous":
-        return run_continuous(args)
-    if args.workload == "trace":
-        return run_trace(args)
-    if args.workload == "attention":
-        return run_attention(args)
-    if args.workload == "latency":
-        return run_latency(args)
-
+def measure_shape(args, shape: str, peaks) -> dict:
+    """Prefill of 2,048 tokens and decode steps of the preset ``shape`` (random weights): the
+    result record of the default workload."""
     from tokamak_amd.config import find_preset
-    from tokamak_amd.kernels import ops
 
-    arch, full = find_preset(args.shape)
-    cfg = dataclasses.replace(full, num_layers=args.layers or full.num_layers)
+    arch, full = find_preset(shape)
+    cfg = arch.shorten(full, args.layers) if args.layers and arch.shorten is not None else full
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
     prompt_tokens = args.prompt if args.context is None else args.context - args.steps
     if prompt_tokens < 1:
-        ap.error("--context must exceed --steps")
+        raise SystemExit("--context must exceed --steps")
     final_context = prompt_tokens + args.steps
     want_points = not args.no_points and args.phase == "all"
     max_batch = max(64 if want_points else 1, args.batch)
-    peaks = None if args.no_peaks else measure_peaks()
     deepest = max(final_context, prompt_tokens + 129) if args.profile else final_context   # (the profiled step sits 129 tokens in)
     pool = max_batch * (-(-(deepest + 1) // PAGE_SIZE) * PAGE_SIZE + PAGE_SIZE)
     longest = max(deepest + 1, PREFILL_TOKENS + 1)
@@ -659,7 +616,7 @@ def main() -> int:
         kernels = profile_kernels(runner, vocab, args.batch, prompt_tokens, key, make_blocker())
 
     sizes = arch.to_json(cfg) if arch.to_json else {}
-    config = {"model": f"{args.shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers}
+    config = {"model": f"{shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers}
     for name, short in (("hidden_size", "hidden_size"), ("num_attention_heads", "heads"),
                         ("num_key_value_heads", "kv_heads"), ("head_dim", "head_dim"),
                         ("intermediate_size", "intermediate_size"), ("vocab_size", "vocab_size")):
@@ -668,7 +625,7 @@ def main() -> int:
     config.update({"global_batch": args.batch, "prompt_tokens": prompt_tokens, "generated_tokens": args.steps,
                    "seq_len": final_context, "page_size": PAGE_SIZE, "repeats": args.repeats,
                    "tuned_products": not args.no_tune, "sampling": "greedy", "parallelism": "single GPU"})
-    what = (f"decode tok/s at batch {args.batch} ({args.shape}-shaped, random weights, {prompt_tokens}-token prompts "
+    what = (f"decode tok/s at batch {args.batch} ({shape}-shaped, random weights, {prompt_tokens}-token prompts "
             f"+ {args.steps} generated); prefill tok/s at {PREFILL_TOKENS} tokens")
     result = {
         "metric": what, "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -703,7 +660,95 @@ def main() -> int:
         result["peaks"] = peaks
     if kernels:
         result["kernels"] = kernels
-    print(json.dumps(result))
+    return result
+
+
+def run_compare(args, peaks) -> int:
+    """Optional extra workload: a design beside the closest model the engine already had, at
+    equal sizes.  ``--pairs a:b,c:d`` names presets; each is measured as the default workload
+    measures ``--shape`` (prefill of 2,048 tokens, decode at ``--batch``; ``--layers`` layers;
+    ``--profile`` adds every kernel's time and its fraction of the roof), one after the other,
+    and one line holds all of them."""
+    import gc
+
+    import torch
+
+    out = {}
+    for pair in args.pairs.split(","):
+        for shape in pair.split(":"):
+            if shape in out:
+                continue
+            record = measure_shape(args, shape, peaks)
+            record.pop("peaks", None)
+            out[shape] = record
+            gc.collect()
+            torch.cuda.empty_cache()
+    rows = []
+    for pair in args.pairs.split(","):
+        new, old = pair.split(":")
+        a, b = out[new], out[old]
+        rows.append({"design": new, "beside": old,
+                     "decode_tok_s": [a["value"], b["value"]],
+                     "decode_hbm_frac": [a.get("roofline", {}).get("frac"), b.get("roofline", {}).get("frac")],
+                     "prefill_tok_s": [a.get("prefill", {}).get("value"), b.get("prefill", {}).get("value")],
+                     "prefill_mfma_frac": [a.get("prefill", {}).get("frac"), b.get("prefill", {}).get("frac")]})
+    print(json.dumps({"metric": "a design beside the closest existing model at equal sizes (decode tok/s, prefill tok/s)",
+                      "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic", "pairs": rows,
+                      "shapes": out, "peaks": peaks}))
+    return 0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256, help="timed decode steps of a pass (the headline workload: 256)")
+    ap.add_argument("--warmup", type=int, default=8, help="untimed decode steps before the timed passes")
+    ap.add_argument("--repeats", type=int, default=3, help="timed passes; the median is reported")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=2048, help="prompt tokens of every request")
+    ap.add_argument("--context", type=int, default=None,
+                    help="instead of --prompt: the timed steps end when each request holds this many tokens")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the microbenchmarks of this GPU's peaks")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="take the library's first algorithm for long portions' products instead of timing its candidates")
+    ap.add_argument("--profile", action="store_true", help="add per-kernel times of one decode and one prefill step")
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
+                    help="run only one part (for an external profiler); the other part's figures are null")
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace", "attention", "latency", "compare"],
+                    help="decode: the headline measurement; continuous: LLM.generate over many requests; "
+                         "trace: the reference's 32-request throughput trace at 1, 4 and 16 running requests; "
+                         "attention: the reference's decode-attention microbenchmark; "
+                         "latency: its single-sequence latency measurement (512 + 128 tokens)")
+    ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
+    ap.add_argument("--shape", default="qwen3-8b",
+                    help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
+    ap.add_argument("--pairs", default="rorosun-0.6b:qwen3-0.6b,rorosun-8b:qwen3-8b",
+                    help="compare workload: NEW:OLD preset pairs, each measured like --shape")
+    ap.add_argument("--requests", type=int, default=256)
+    ap.add_argument("--max-batch", type=int, default=64)
+    ap.add_argument("--prompt-tokens", default="32,1024", help="continuous workload: MIN,MAX prompt length")
+    ap.add_argument("--output-tokens", default="16,256", help="continuous workload: MIN,MAX output length")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+    if args.workload == "continuous":
+        return run_continuous(args)
+    if args.workload == "trace":
+        return run_trace(args)
+    if args.workload == "attention":
+        return run_attention(args)
+    if args.workload == "latency":
+        return run_latency(args)
+
+    peaks = None if args.no_peaks else measure_peaks()
+    if args.workload == "compare":
+        return run_compare(args, peaks)
+    print(json.dumps(measure_shape(args, args.shape, peaks)))
     return 0
 
 

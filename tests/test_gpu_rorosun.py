@@ -200,7 +200,9 @@ def test_pooled_window_attention_alone(dtype, a):
     pages = 40
     store = SlotStore(0, page, {
         "k": torch.full((pages, left["kv_heads"] * left["dim"] * page), float("nan"), dtype=dtype, device=DEV),
-        "v": torch.full((pages, left["kv_heads"] * left["vdim"] * page), float("nan"), dtype=dtype, device=DEV)})
+        "v": torch.full((pages, left["kv_heads"] * left["vdim"] * page), float("nan"), dtype=dtype, device=DEV),
+        **{name: torch.full((pages, array.elems_per_token * page), float("nan"), dtype=array.dtype, device=DEV)
+           for name, array in part.cache_request().arrays if name.endswith("_pool")}})
     table = [(7 * i + 3) % pages for i in range(-(-T // page))]
     assert len(set(table)) == len(table)
     got, at = [], 0

@@ -24,7 +24,9 @@ class Architecture:
     the typed config back as a ``config.json`` dict (used by the random-weights
     folder writer).  ``presets``: named typed configs (shapes for the
     random-weights mode of the command line and the benchmark).  ``chat_prompt``:
-    user text -> prompt text, used when a model folder has no chat template."""
+    user text -> prompt text, used when a model folder has no chat template.
+    ``shorten``: (typed config, n) -> the same model with its first n layers only (the
+    benchmark measures a few layers of a wide shape)."""
 
     name: str
     parse: Callable[[dict[str, Any], tuple[int, ...]], Any]
@@ -32,6 +34,7 @@ class Architecture:
     to_json: Callable[[Any], dict[str, Any]] | None = None
     presets: Mapping[str, Any] = field(default_factory=dict)
     chat_prompt: Callable[[str], str] | None = None
+    shorten: Callable[[Any, int], Any] | None = None
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}

@@ -8,6 +8,12 @@
 //     w'_h(e) = sum_g talk[h, g] w_g(e),
 // and head h applies w'_h to the values of its own kv head.
 //
+// The means live in pages of their own arrays (float32): block b's mean is elements
+// [b * W, (b + 1) * W) of the request's flat pooled array, which has ceil(W / pool) elements for
+// every position, so a block's mean lies in pages the request already owns when the block is
+// complete.  pool_blocks writes the mean of every block that a step completes, summing the
+// block's cached rows in position order.
+//
 // bias_norm_store: the q/k/v projection's output plus biases; q and k each divided by the root
 //   mean square of their WHOLE row (all heads) and multiplied by a weight per coordinate; q goes
 //   out, k and v into the request's pages.  Page layout: [page][token in page][G * dim].
@@ -73,13 +79,49 @@ __global__ __launch_bounds__(256) void bias_norm_store_kernel(
   }
 }
 
+// element c of block b's mean in a pooled array with E elements a position
+__device__ __forceinline__ size_t pooled_at(const int* __restrict__ table, int b, int c, int width, int E,
+                                            int page_size) {
+  const size_t flat = (size_t)b * width + c;
+  const size_t per_page = (size_t)page_size * E;
+  return (size_t)table[flat / per_page] * per_page + flat % per_page;
+}
+
+// a token that completes a block of `pool` positions writes the block's mean key and value
+template <typename T>
+__global__ __launch_bounds__(256) void pool_blocks_kernel(
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache, float* __restrict__ k_pool,
+    float* __restrict__ v_pool, const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ tables, int table_width, int KW, int VW, int KE, int VE, int pool, int page_size) {
+  const int n = blockIdx.x;
+  const int pos = positions[n];
+  if ((pos + 1) % pool != 0) return;
+  const int b = pos / pool;
+  const int* table = tables + (size_t)req_of_token[n] * table_width;
+  const float inv = 1.f / (float)pool;
+  for (int c = threadIdx.x; c < KW + VW; c += blockDim.x) {
+    const bool key = c < KW;
+    const int width = key ? KW : VW, col = key ? c : c - KW;
+    const T* cache = key ? k_cache : v_cache;
+    float s = 0.f;
+    for (int t = 0; t < pool; ++t) {
+      const int p = b * pool + t;
+      s += Elem<T>::load(cache + ((size_t)table[p / page_size] * page_size + p % page_size) * width + col);
+    }
+    if (key) k_pool[pooled_at(table, b, col, KW, KE, page_size)] = s * inv;
+    else v_pool[pooled_at(table, b, col, VW, VE, page_size)] = s * inv;
+  }
+}
+
 struct PoolArgs {
   const int* positions;
   const int* req_of_token;
   const int* q_start;
   const int* tables;
   const float* talk;
-  int table_width, N, H, G, dim, vdim, size, pool, page_size, TQ, CH;
+  const float* k_pool;
+  const float* v_pool;
+  int table_width, N, H, G, dim, vdim, size, pool, page_size, TQ, CH, KE, VE;
   float scale;
 };
 
@@ -87,21 +129,15 @@ constexpr int kAcc = 16;   // outputs a thread accumulates: TQ * H * vdim <= kAc
 
 // rows [e0, e0 + ne) of a chunk: entry e < NB is block e's mean, else token j0 + (e - NB)
 template <typename T>
-__device__ __forceinline__ void stage(const T* __restrict__ cache, const int* __restrict__ table, float* dst,
-                                      int width, int padded, int e0, int ne, int NB, int j0, int pool,
-                                      int page_size) {
-  const float inv = 1.f / (float)pool;
+__device__ __forceinline__ void stage(const T* __restrict__ cache, const float* __restrict__ pooled,
+                                      const int* __restrict__ table, float* dst, int width, int padded, int e0,
+                                      int ne, int NB, int j0, int E, int page_size) {
   for (int idx = threadIdx.x; idx < ne * width; idx += blockDim.x) {
     const int e = idx / width, c = idx - e * width;
     const int entry = e0 + e;
     float v;
     if (entry < NB) {
-      float s = 0.f;
-      for (int t = 0; t < pool; ++t) {
-        const int p = entry * pool + t;
-        s += Elem<T>::load(cache + ((size_t)table[p / page_size] * page_size + p % page_size) * width + c);
-      }
-      v = s * inv;
+      v = pooled[pooled_at(table, entry, c, width, E, page_size)];
     } else {
       const int p = j0 + entry - NB;
       v = Elem<T>::load(cache + ((size_t)table[p / page_size] * page_size + p % page_size) * width + c);
@@ -156,8 +192,8 @@ __global__ void pooled_window_attention_kernel(const T* __restrict__ q, const T*
       for (int e0 = 0; e0 < E; e0 += CH) {
         const int ne = min(CH, E - e0);
         __syncthreads();
-        stage<T>(k_cache, table, Ks, KW, KP, e0, ne, NB, j0, a.pool, a.page_size);
-        if (pass == 1) stage<T>(v_cache, table, Vs, VW, VP, e0, ne, NB, j0, a.pool, a.page_size);
+        stage<T>(k_cache, a.k_pool, table, Ks, KW, KP, e0, ne, NB, j0, a.KE, a.page_size);
+        if (pass == 1) stage<T>(v_cache, a.v_pool, table, Vs, VW, VP, e0, ne, NB, j0, a.VE, a.page_size);
         __syncthreads();
         // scores, or (second pass) normalised weights
         for (int idx = tid; idx < tq * H * ne; idx += nthreads) {
@@ -260,6 +296,23 @@ TK_API int tk_bias_norm_store(int dtype, const void* qkv, int in_f32, int parts,
   return launch_status();
 }
 
+// k_pool / v_pool: float32 paged arrays with KE / VE elements a position (>= ceil(width / pool))
+TK_API int tk_pool_blocks(int dtype, const void* k_cache, const void* v_cache, float* k_pool, float* v_pool,
+                          const int* positions, const int* req_of_token, const int* tables, int table_width, int N,
+                          int KW, int VW, int KE, int VE, int pool, int page_size, hipStream_t stream) {
+  if (N <= 0) return 0;
+  if (pool < 1 || page_size < 1 || (long)KE * pool < KW || (long)VE * pool < VW) return -2;
+  if (dtype == 0)
+    pool_blocks_kernel<float><<<N, 256, 0, stream>>>((const float*)k_cache, (const float*)v_cache, k_pool, v_pool,
+                                                     positions, req_of_token, tables, table_width, KW, VW, KE, VE,
+                                                     pool, page_size);
+  else
+    pool_blocks_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)k_cache, (const bf16_t*)v_cache, k_pool, v_pool,
+                                                      positions, req_of_token, tables, table_width, KW, VW, KE, VE,
+                                                      pool, page_size);
+  return launch_status();
+}
+
 // LDS bytes of a launch with tiles of TQ rows and chunks of CH entries
 TK_API long tk_pooled_window_lds(int H, int G, int dim, int vdim, int TQ, int CH) {
   const long floats = (long)TQ * H * dim + (long)CH * (G * dim + 1) + (long)CH * (G * vdim + 1) +
@@ -268,18 +321,20 @@ TK_API long tk_pooled_window_lds(int H, int G, int dim, int vdim, int TQ, int CH
 }
 
 TK_API int tk_pooled_window_attention(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                                      const float* k_pool, const float* v_pool, int KE, int VE,
                                       void* out, const int* positions, const int* req_of_token,
                                       const int* q_start, const int* tables, int table_width, const float* talk,
                                       int N, int H, int G, int dim, int vdim, int size, int pool, int page_size,
                                       int TQ, int CH, int threads, float scale, hipStream_t stream) {
   if (N <= 0) return 0;
   if (H < 1 || G < 1 || H % G || dim < 1 || vdim < 1 || size < 1 || pool < 1 || page_size < 1 || TQ < 1 || CH < 1 ||
-      threads % kWave || threads < kWave || threads > 1024 || (long)TQ * H * vdim > (long)kAcc * threads)
+      threads % kWave || threads < kWave || threads > 1024 || (long)TQ * H * vdim > (long)kAcc * threads ||
+      (long)KE * pool < (long)G * dim || (long)VE * pool < (long)G * vdim)
     return -2;
   const long lds = tk_pooled_window_lds(H, G, dim, vdim, TQ, CH);
   if (lds > 160 * 1024) return -3;
-  PoolArgs a{positions, req_of_token, q_start, tables, talk, table_width, N, H, G, dim, vdim,
-             size, pool, page_size, TQ, CH, scale};
+  PoolArgs a{positions, req_of_token, q_start, tables, talk, k_pool, v_pool, table_width, N, H, G, dim, vdim,
+             size, pool, page_size, TQ, CH, KE, VE, scale};
   const unsigned blocks = (unsigned)((N + TQ - 1) / TQ);
   // the most LDS asked for so far is allowed once per kernel (not at every launch: a launch
   // may be recorded into a graph, whose first, eager run has then already raised the limit)
@@ -302,4 +357,5 @@ TK_API int tk_pooled_window_attention(int dtype, const void* q, const void* k_ca
 }
 
 TK_SLOTS(tk_bias_norm_store)
+TK_SLOTS(tk_pool_blocks)
 TK_SLOTS(tk_pooled_window_attention)

@@ -182,7 +182,10 @@ _SIGS = {
         "tk_bias_norm_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                c_int, c_float, c_int, c_void_p],
-        "tk_pooled_window_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        "tk_pool_blocks": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_pooled_window_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                       c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_float, c_void_p],
     },
@@ -504,6 +507,37 @@ def bias_norm_store(qkv: torch.Tensor, bias: torch.Tensor, q_weight: torch.Tenso
         v_width, page_size, float(eps), int(bool(store)), _stream()), "bias_norm_store")
 
 
+def pooled_elems(width: int, pool: int) -> int:
+    """Elements a position of a pooled array: block b's mean of ``width`` numbers is elements
+    [b * width, (b + 1) * width) of the request's flat array, which therefore lies in pages the
+    request owns once the block's ``pool`` positions are stored."""
+    return -(-width // pool)
+
+
+def _pooled_arrays(k_pool, v_pool, k_cache, k_width, v_width, pool, page_size):
+    _need(k_pool.dtype == torch.float32 and v_pool.dtype == torch.float32, "pooled arrays are float32")
+    _need(k_pool.shape[0] == k_cache.shape[0] == v_pool.shape[0] and k_pool.shape[1] % page_size == 0
+          and v_pool.shape[1] % page_size == 0, "pooled arrays do not have the page layout")
+    ke, ve = k_pool.shape[1] // page_size, v_pool.shape[1] // page_size
+    _need(ke * pool >= k_width and ve * pool >= v_width, "pooled arrays are too narrow for a block's mean")
+    return ke, ve
+
+
+def pool_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                positions: torch.Tensor, req_of_token: torch.Tensor, tables: torch.Tensor, n: int, *,
+                k_width: int, v_width: int, pool: int, page_size: int) -> None:
+    """Every token of the step that completes a block of ``pool`` positions writes the means of
+    the block's cached keys and values (summed in position order, float32) into the pooled arrays."""
+    _gpu(k_cache, v_cache, k_pool, v_pool, positions, req_of_token, tables)
+    _need(k_cache.dtype == v_cache.dtype and k_cache.shape[1] == k_width * page_size
+          and v_cache.shape[1] == v_width * page_size, "cache arrays do not have the page layout")
+    _need(positions.numel() >= n and req_of_token.numel() >= n and tables.dim() == 2, "step descriptor arrays are too short")
+    ke, ve = _pooled_arrays(k_pool, v_pool, k_cache, k_width, v_width, pool, page_size)
+    _check(_fn("attention_pooled", "tk_pool_blocks")(
+        _code(k_cache.dtype), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool), _p(positions), _p(req_of_token),
+        _p(tables), tables.shape[1], n, k_width, v_width, ke, ve, pool, page_size, _stream()), "pool_blocks")
+
+
 POOLED_LDS_BYTES = 144 * 1024      # of a CU's 160 KB
 POOLED_ACC = 16                    # outputs a thread of the attention kernel accumulates
 
@@ -528,13 +562,15 @@ def pooled_window_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, l
     return rows, chunk, threads
 
 
-def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,
-                            batch, talk: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
+def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torch.Tensor,
+                            v_pool: torch.Tensor, tables: torch.Tensor, batch, talk: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                             dim: int, vdim: int, window: int, pool: int, page_size: int, scale: float) -> None:
     """Attention of every row of the step over its request's pages: the last ``window``
     positions one by one, complete blocks of ``pool`` positions behind them by the means of
-    their keys and values, one softmax over both, the heads' weights mixed by ``talk`` [H, H]."""
-    _gpu(q, k_cache, v_cache, tables, talk, out)
+    their keys and values (``k_pool``, ``v_pool``, written by ``pool_blocks``), one softmax over
+    both, the heads' weights mixed by ``talk`` [H, H]."""
+    _gpu(q, k_cache, v_cache, k_pool, v_pool, tables, talk, out)
+    ke, ve = _pooled_arrays(k_pool, v_pool, k_cache, num_kv_heads * dim, num_kv_heads * vdim, pool, page_size)
     n = q.shape[0]
     dtype = q.dtype
     _need(q.shape == (n, num_heads * dim) and out.shape == (n, num_heads * vdim) and out.dtype == dtype, "q/out shapes disagree")
@@ -546,10 +582,21 @@ def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
           "block tables do not match the step")
     _need(-(-batch.max_seq_len // page_size) <= tables.shape[1], "a block table is shorter than its request")
     rows, chunk, threads = pooled_window_plan(num_heads, num_kv_heads, dim, vdim, batch.max_q_len)
-    _note(f"{n}x{num_heads}x{dim}", 0.0, 0.0)
+    if _profile is not None:
+        # the least a step has to move: every cached position of every request once, queries in,
+        # results out; and two multiply-adds per head, channel and visible entry
+        elem = q.element_size()
+        entries = 0
+        for q_len, ctx in zip(batch.q_lens, batch.ctx_lens):
+            for i in range(ctx, ctx + q_len):
+                entries += min(i + 1, window) + max(0, (i - window - (pool - 1)) // pool + 1 if i - window >= pool - 1 else 0)
+        # (a request's window of rows in the cache's type, its blocks' means in float32)
+        cached = sum(min(c + ql, window + ql - 1) * elem + (c + ql) // pool * 4 for c, ql in zip(batch.ctx_lens, batch.q_lens))
+        _note(f"{n}x{num_heads}x{dim}", cached * num_kv_heads * (dim + vdim) + n * num_heads * (dim + vdim) * elem,
+              2.0 * num_heads * (dim + vdim) * entries)
     _check(_fn("attention_pooled", "tk_pooled_window_attention")(
-        _code(dtype), _p(q), _p(k_cache), _p(v_cache), _p(out), _p(batch.positions), _p(batch.req_of_token),
-        _p(batch.q_start), _p(tables), tables.shape[1], _p(talk), n, num_heads, num_kv_heads, dim, vdim, window, pool,
+        _code(dtype), _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool), ke, ve, _p(out), _p(batch.positions),
+        _p(batch.req_of_token), _p(batch.q_start), _p(tables), tables.shape[1], _p(talk), n, num_heads, num_kv_heads, dim, vdim, window, pool,
         page_size, rows, chunk, threads, float(scale), _stream()), "pooled_window_attention")
 
 

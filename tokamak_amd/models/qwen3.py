@@ -9,7 +9,7 @@ the embedding matrix.  No biases anywhere.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Any
 
 from tokamak_amd.config.model_config import (
@@ -211,5 +211,9 @@ PRESETS = {
 }
 
 
+def shorten(cfg: Qwen3Config, num_layers: int) -> Qwen3Config:
+    return replace(cfg, num_layers=min(num_layers, cfg.num_layers))
+
+
 register_architecture(Architecture(name=NAME, parse=parse, plan=plan, to_json=to_config_json,
-                                   presets=PRESETS, chat_prompt=chat_prompt))
+                                   presets=PRESETS, chat_prompt=chat_prompt, shorten=shorten))

@@ -18,7 +18,7 @@ Tensor names: ``embed``, ``l<i>.norm1``, ``l<i>.norm2``, ``l<i>.mix.left.*``, ``
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Any
 
 from tokamak_amd.config.model_config import LayerCall, LayerSpec, ModelPlan, PartSpec, SubPart
@@ -217,4 +217,9 @@ PRESETS = {
 }
 
 
-register_architecture(Architecture(name=NAME, parse=parse, plan=plan, to_json=to_config_json, presets=PRESETS))
+def shorten(cfg: RorosunConfig, num_layers: int) -> RorosunConfig:
+    return replace(cfg, layers=cfg.layers[:num_layers])
+
+
+register_architecture(Architecture(name=NAME, parse=parse, plan=plan, to_json=to_config_json, presets=PRESETS,
+                                   shorten=shorten))

@@ -7,7 +7,7 @@ import torch
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
 from tokamak_amd.kernels.linear import linear
-from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer, PositionData
+from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer, PagedArray, PositionData
 from tokamak_amd.weights.spec import TensorSpec
 
 
@@ -25,8 +25,10 @@ class PooledWindowAttention(Mixer):
     values of kv head a // (num_heads / num_kv_heads).  Keys have ``head_dim`` channels, values
     ``value_dim``.  Tensors: q, k, v (matrices) with q.b, k.b, v.b, q.norm, k.norm, talk, o.
 
-    Every position's key and value stay in the pages (the blocks are pooled from them when they
-    are read), so the cache group keeps everything.
+    The cache holds four paged arrays: keys and values of every position in the compute dtype,
+    and the blocks' mean keys and values in float32 (``pool`` times narrower), written by the
+    token that completes a block from the rows the cache holds.  A query then reads ``window``
+    rows and one mean per block behind them, not the whole context.
     """
 
     capturable = True
@@ -74,7 +76,9 @@ class PooledWindowAttention(Mixer):
         self.o = fetch(prefix + "o")
 
     def cache_request(self) -> CacheRequest:
-        return CacheRequest.of(window=None, k=self.k_width, v=self.v_width)
+        return CacheRequest.of(window=None, k=self.k_width, v=self.v_width,
+                               k_pool=PagedArray(ops.pooled_elems(self.k_width, self.pool), torch.float32),
+                               v_pool=PagedArray(ops.pooled_elems(self.v_width, self.pool), torch.float32))
 
     def pair_flops(self) -> float:
         return 2.0 * self.num_heads * (self.head_dim + self.value_dim)
@@ -89,8 +93,13 @@ class PooledWindowAttention(Mixer):
         ops.bias_norm_store(qkv, self.bias, self.q_norm, self.k_norm, batch.positions, batch.req_of_token, tables, q,
                             store.arrays["k"], store.arrays["v"], q_width=self.q_width, k_width=self.k_width,
                             v_width=self.v_width, page_size=store.page_size, eps=self.norm_eps, store=writes_cache)
+        if writes_cache:
+            ops.pool_blocks(store.arrays["k"], store.arrays["v"], store.arrays["k_pool"], store.arrays["v_pool"],
+                            batch.positions, batch.req_of_token, tables, n, k_width=self.k_width,
+                            v_width=self.v_width, pool=self.pool, page_size=store.page_size)
         attended = torch.empty((n, self.num_heads * self.value_dim), dtype=self.dtype, device=h.device)
-        ops.pooled_window_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, self.talk, attended,
+        ops.pooled_window_attention(q, store.arrays["k"], store.arrays["v"], store.arrays["k_pool"],
+                                    store.arrays["v_pool"], tables, batch, self.talk, attended,
                                     num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, dim=self.head_dim,
                                     vdim=self.value_dim, window=self.window, pool=self.pool,
                                     page_size=store.page_size, scale=self.softmax_scale)
