@@ -273,6 +273,346 @@ __global__ void pooled_window_attention_kernel(const T* __restrict__ q, const T*
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// The same attention in three kernels that fill the GPU whatever the step's shape: a block
+// takes up to TQ consecutive rows of one request, ONE kv head and one share of the entries.
+//   scores:  a lane an entry: its key row (or block mean) against the queries of the kv head's
+//            query heads; raw scores to memory [row][entry][head], and every (row, head)'s
+//            maximum and sum of exponentials over the share.
+//   values:  merges the shares' statistics of ALL heads, turns the scores of its entries into
+//            normalised weights, mixes them for its own query heads, and applies them to its
+//            kv head's values (a wave an entry, a lane a channel); float32 partial outputs.
+//   merge:   adds the shares' partial outputs.
+constexpr int kGroupMax = 16;   // query heads a kv head
+constexpr int kTileMax = 8;     // rows a block
+constexpr int kPairMax = 32;    // rows times query heads a lane accumulates in the score kernel
+constexpr int kChanMax = 4;     // value channels a lane: vdim <= 256
+constexpr int kSplitThreads = 256;
+
+struct SplitArgs {
+  const int* positions;
+  const int* req_of_token;
+  const int* q_start;
+  const int* tables;
+  const float* talk;
+  const float* k_pool;
+  const float* v_pool;
+  float* scores;     // [N][Emax][H]
+  float* part_m;     // [N][H][S]
+  float* part_l;     // [N][H][S]
+  float* part_o;     // [S][N][H * vdim]
+  int table_width, N, H, G, dim, vdim, size, pool, page_size, TQ, S, Emax, KE, VE;
+  float scale;
+};
+
+struct Segment {
+  int row, tq, i0, NB, j0, E;
+  const int* table;
+};
+
+// the rows [row, seg_end) of one request inside a block's tile, and the entries they see together
+__device__ __forceinline__ Segment segment_at(const SplitArgs& a, int row, int row_end) {
+  Segment g;
+  const int r = a.req_of_token[row];
+  g.row = row;
+  g.tq = min(row_end, a.q_start[r + 1]) - row;
+  g.i0 = a.positions[row];
+  const int i_last = g.i0 + g.tq - 1;
+  const int behind = i_last - a.size - (a.pool - 1);
+  g.NB = behind >= 0 ? behind / a.pool + 1 : 0;
+  g.j0 = max(0, g.i0 - a.size + 1);
+  g.E = g.NB + i_last - g.j0 + 1;
+  g.table = a.tables + (size_t)r * a.table_width;
+  return g;
+}
+
+__device__ __forceinline__ bool entry_seen(const SplitArgs& a, const Segment& g, int entry, int i) {
+  if (entry < g.NB) return entry * a.pool + a.pool - 1 <= i - a.size;
+  const int j = g.j0 + entry - g.NB;
+  return j <= i && i - j < a.size;
+}
+
+template <typename T>
+__device__ __forceinline__ float entry_value(const T* __restrict__ cache, const float* __restrict__ pooled,
+                                             const Segment& g, int entry, int col, int width, int E, int page_size) {
+  if (entry < g.NB) return pooled[pooled_at(g.table, entry, col, width, E, page_size)];
+  const int p = g.j0 + entry - g.NB;
+  return Elem<T>::load(cache + ((size_t)g.table[p / page_size] * page_size + p % page_size) * width + col);
+}
+
+__device__ __forceinline__ void load8(const float* p, float* o) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float* o) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSplitThreads) void pooled_scores_kernel(const T* __restrict__ q,
+                                                                      const T* __restrict__ k_cache, SplitArgs a) {
+  extern __shared__ float lds[];
+  const int group = a.H / a.G, dim = a.dim, KW = a.G * a.dim;
+  const int c = blockIdx.y, split = blockIdx.z;
+  float* qs = lds;                                   // [TQ][group][dim]
+  float* red = qs + a.TQ * group * dim;              // [waves][TQ * group][2]
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  constexpr int kWaves = kSplitThreads / kWave;
+  const int row_end = min(a.N, (int)(blockIdx.x + 1) * a.TQ);
+  int row = blockIdx.x * a.TQ;
+  while (row < row_end) {
+    const Segment g = segment_at(a, row, row_end);
+    const int pairs = g.tq * group;
+    __syncthreads();
+    for (int i = tid; i < pairs * dim; i += kSplitThreads) {
+      const int x = i % dim, tg = i / dim, t = tg / group, h = tg % group;
+      qs[i] = Elem<T>::load(q + (size_t)(g.row + t) * a.H * dim + (c * group + h) * dim + x);
+    }
+    __syncthreads();
+    const int e_lo = (int)((long)g.E * split / a.S), e_hi = (int)((long)g.E * (split + 1) / a.S);
+    // 16-byte loads where every row starts on a 16-byte border
+    const bool vec = dim % 8 == 0 && KW % 8 == 0;
+    const bool pvec = vec && ((long)a.page_size * a.KE) % 4 == 0;
+    float m[kPairMax], l[kPairMax];
+#pragma unroll
+    for (int p = 0; p < kPairMax; ++p) {
+      m[p] = -INFINITY;
+      l[p] = 0.f;
+    }
+    for (int entry = e_lo + tid; entry < e_hi; entry += kSplitThreads) {
+      float acc[kPairMax];
+#pragma unroll
+      for (int p = 0; p < kPairMax; ++p) acc[p] = 0.f;
+      // the entry's row for this kv head: a cache row, a block mean inside one page, or (a mean
+      // across a page border) neither, and then element by element
+      const T* rowp = nullptr;
+      const float* poolp = nullptr;
+      if (entry < g.NB) {
+        const size_t first = (size_t)entry * KW + (size_t)c * dim, per_page = (size_t)a.page_size * a.KE;
+        if (first % per_page + dim <= per_page) poolp = a.k_pool + (size_t)g.table[first / per_page] * per_page + first % per_page;
+      } else {
+        const int p = g.j0 + entry - g.NB;
+        rowp = k_cache + ((size_t)g.table[p / a.page_size] * a.page_size + p % a.page_size) * KW + (size_t)c * dim;
+      }
+      for (int x0 = 0; x0 < dim; x0 += 8) {
+        float kx[8];
+        if (rowp != nullptr && vec) {
+          load8(rowp + x0, kx);
+        } else if (poolp != nullptr && pvec) {
+          load8(poolp + x0, kx);
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int x = x0 + u;
+            kx[u] = x >= dim ? 0.f
+                    : rowp != nullptr ? Elem<T>::load(rowp + x)
+                    : poolp != nullptr ? poolp[x]
+                                       : entry_value<T>(k_cache, a.k_pool, g, entry, c * dim + x, KW, a.KE, a.page_size);
+          }
+        }
+        const int left = min(8, dim - x0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (u < left) {
+#pragma unroll
+            for (int p = 0; p < kPairMax; ++p)
+              if (p < pairs) acc[p] = fmaf(qs[p * dim + x0 + u], kx[u], acc[p]);
+          }
+        }
+      }
+#pragma unroll
+      for (int p = 0; p < kPairMax; ++p) {
+        if (p < pairs) {
+          const int t = p / group, h = p % group;
+          const bool seen = entry_seen(a, g, entry, g.i0 + t);
+          const float sc = seen ? acc[p] * a.scale : -INFINITY;
+          a.scores[((size_t)(g.row + t) * a.Emax + entry) * a.H + c * group + h] = sc;
+          if (seen) {
+            const float m_new = fmaxf(m[p], sc);
+            l[p] = l[p] * expf(m[p] - m_new) + expf(sc - m_new);     // (exp(-inf) = 0 the first time)
+            m[p] = m_new;
+          }
+        }
+      }
+    }
+    // the block's maximum and sum of every (row, head): lanes, then waves
+#pragma unroll
+    for (int p = 0; p < kPairMax; ++p) {
+      if (p < pairs) {
+        const float m_all = wave_max(m[p]);
+        const float l_all = wave_sum(m[p] > -INFINITY ? l[p] * expf(m[p] - m_all) : 0.f);
+        if (lane == 0) {
+          red[(wave * kPairMax + p) * 2] = m_all;
+          red[(wave * kPairMax + p) * 2 + 1] = l_all;
+        }
+      }
+    }
+    __syncthreads();
+    for (int p = tid; p < pairs; p += kSplitThreads) {
+      float m_all = -INFINITY;
+      for (int w = 0; w < kWaves; ++w) m_all = fmaxf(m_all, red[(w * kPairMax + p) * 2]);
+      float l_all = 0.f;
+      for (int w = 0; w < kWaves; ++w) {
+        const float mw = red[(w * kPairMax + p) * 2];
+        if (mw > -INFINITY) l_all += red[(w * kPairMax + p) * 2 + 1] * expf(mw - m_all);
+      }
+      const int t = p / group, h = p % group;
+      const size_t at = ((size_t)(g.row + t) * a.H + c * group + h) * a.S + split;
+      a.part_m[at] = m_all;
+      a.part_l[at] = l_all;
+    }
+    row += g.tq;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* __restrict__ v_cache,
+                                                                      T* __restrict__ out, SplitArgs a) {
+  extern __shared__ float lds[];
+  const int H = a.H, group = a.H / a.G, vdim = a.vdim, VW = a.G * a.vdim;
+  const int c = blockIdx.y, split = blockIdx.z;
+  constexpr int kWaves = kSplitThreads / kWave;
+  float* mh = lds;                                   // [TQ][H]  maximum of every head
+  float* il = mh + a.TQ * H;                         // [TQ][H]  1 / sum
+  float* tk_ = il + a.TQ * H;                        // [group][H]
+  float* wm = tk_ + group * H;                       // [TQ * group][kSplitThreads] mixed weights of a chunk
+  float* red = wm + a.TQ * group * kSplitThreads;    // [waves][TQ * group][vdim]
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  for (int i = tid; i < group * H; i += kSplitThreads) tk_[i] = a.talk[(size_t)(c * group + i / H) * H + i % H];
+  const int row_end = min(a.N, (int)(blockIdx.x + 1) * a.TQ);
+  int row = blockIdx.x * a.TQ;
+  while (row < row_end) {
+    const Segment g = segment_at(a, row, row_end);
+    const int pairs = g.tq * group;
+    __syncthreads();
+    for (int i = tid; i < g.tq * H; i += kSplitThreads) {
+      const size_t at = ((size_t)(g.row + i / H) * H + i % H) * a.S;
+      float m_all = -INFINITY;
+      for (int s = 0; s < a.S; ++s) m_all = fmaxf(m_all, a.part_m[at + s]);
+      float l_all = 0.f;
+      for (int s = 0; s < a.S; ++s) {
+        const float ms = a.part_m[at + s];
+        if (ms > -INFINITY) l_all += a.part_l[at + s] * expf(ms - m_all);
+      }
+      mh[i] = m_all;
+      il[i] = 1.f / l_all;
+    }
+    __syncthreads();
+    const int e_lo = (int)((long)g.E * split / a.S), e_hi = (int)((long)g.E * (split + 1) / a.S);
+    float acc[kPairMax][kChanMax];
+#pragma unroll
+    for (int p = 0; p < kPairMax; ++p)
+#pragma unroll
+      for (int d = 0; d < kChanMax; ++d) acc[p][d] = 0.f;
+    for (int e0 = e_lo; e0 < e_hi; e0 += kSplitThreads) {
+      const int ne = min(kSplitThreads, e_hi - e0);
+      __syncthreads();            // the chunk before is applied
+      if (tid < ne) {
+        for (int t = 0; t < g.tq; ++t) {
+          const float* sc = a.scores + ((size_t)(g.row + t) * a.Emax + e0 + tid) * H;
+          float mixed[kGroupMax];
+#pragma unroll
+          for (int h = 0; h < kGroupMax; ++h) mixed[h] = 0.f;
+          for (int gh = 0; gh < H; ++gh) {
+            const float s = sc[gh];
+            const float w = s > -INFINITY ? expf(s - mh[t * H + gh]) * il[t * H + gh] : 0.f;
+#pragma unroll
+            for (int h = 0; h < kGroupMax; ++h)
+              if (h < group) mixed[h] = fmaf(tk_[h * H + gh], w, mixed[h]);
+          }
+#pragma unroll
+          for (int h = 0; h < kGroupMax; ++h)
+            if (h < group) wm[(t * group + h) * kSplitThreads + tid] = mixed[h];
+        }
+      }
+      __syncthreads();
+      for (int e = wave; e < ne; e += kWaves) {
+        float v[kChanMax];
+#pragma unroll
+        for (int d = 0; d < kChanMax; ++d) {
+          const int x = lane + d * kWave;
+          v[d] = x < vdim ? entry_value<T>(v_cache, a.v_pool, g, e0 + e, c * vdim + x, VW, a.VE, a.page_size) : 0.f;
+        }
+#pragma unroll
+        for (int p = 0; p < kPairMax; ++p) {
+          if (p < pairs) {
+            const float w = wm[p * kSplitThreads + e];
+#pragma unroll
+            for (int d = 0; d < kChanMax; ++d) acc[p][d] = fmaf(w, v[d], acc[p][d]);
+          }
+        }
+      }
+    }
+    // add the waves' sums
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < kPairMax; ++p) {
+      if (p < pairs) {
+#pragma unroll
+        for (int d = 0; d < kChanMax; ++d) {
+          const int x = lane + d * kWave;
+          if (x < vdim) red[(wave * pairs + p) * vdim + x] = acc[p][d];
+        }
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < pairs * vdim; i += kSplitThreads) {
+      float sum = 0.f;
+      for (int w = 0; w < kWaves; ++w) sum += red[(size_t)w * pairs * vdim + i];
+      const int x = i % vdim, p = i / vdim, t = p / group, h = p % group;
+      const size_t at = (size_t)(g.row + t) * H * vdim + (c * group + h) * vdim + x;
+      if (a.S == 1) Elem<T>::store(out + at, sum);
+      else a.part_o[(size_t)split * a.N * H * vdim + at] = sum;
+    }
+    row += g.tq;
+  }
+}
+
+template <typename T>
+__global__ void pooled_merge_kernel(const float* __restrict__ part_o, T* __restrict__ out, int S, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float sum = 0.f;
+  for (int s = 0; s < S; ++s) sum += part_o[(size_t)s * total + idx];
+  Elem<T>::store(out + idx, sum);
+}
+
+template <typename T>
+int launch_split(const void* q, const void* k_cache, const void* v_cache, void* out, const SplitArgs& a,
+                 hipStream_t stream) {
+  const int group = a.H / a.G;
+  const dim3 grid((a.N + a.TQ - 1) / a.TQ, a.G, a.S);
+  const size_t lds_a = ((size_t)a.TQ * group * a.dim + (kSplitThreads / kWave) * kPairMax * 2) * 4;
+  const size_t lds_b = ((size_t)2 * a.TQ * a.H + (size_t)group * a.H + (size_t)a.TQ * group * kSplitThreads +
+                        (size_t)(kSplitThreads / kWave) * a.TQ * group * a.vdim) * 4;
+  if (lds_a > 150 * 1024 || lds_b > 150 * 1024) return -3;
+  static bool allowed = false;      // (per instantiation: once per storage type)
+  if (!allowed) {
+    hipError_t err = hipFuncSetAttribute((const void*)pooled_scores_kernel<T>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (err == hipSuccess)
+      err = hipFuncSetAttribute((const void*)pooled_values_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
+    if (err != hipSuccess) return (int)err;
+    allowed = true;
+  }
+  pooled_scores_kernel<T><<<grid, kSplitThreads, lds_a, stream>>>((const T*)q, (const T*)k_cache, a);
+  pooled_values_kernel<T><<<grid, kSplitThreads, lds_b, stream>>>((const T*)v_cache, (T*)out, a);
+  if (a.S > 1) {
+    const size_t total = (size_t)a.N * a.H * a.vdim;
+    pooled_merge_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(a.part_o, (T*)out, a.S, total);
+  }
+  return launch_status();
+}
+
 }  // namespace
 
 // qkv: [N, QW + KW + VW] (QW alone if !store) in dtype, or float32 / float32 partial sums.
@@ -356,6 +696,27 @@ TK_API int tk_pooled_window_attention(int dtype, const void* q, const void* k_ca
   return launch_status();
 }
 
+// The three-kernel form.  scores [N, Emax, H], part_m / part_l [N, H, S], part_o [S, N, H * vdim]
+// (unused if S == 1) are float32 scratch; Emax bounds the entries any tile of TQ rows sees.
+TK_API int tk_pooled_window_attention_split(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                                            const float* k_pool, const float* v_pool, int KE, int VE, void* out,
+                                            const int* positions, const int* req_of_token, const int* q_start,
+                                            const int* tables, int table_width, const float* talk, float* scores,
+                                            float* part_m, float* part_l, float* part_o, int N, int H, int G,
+                                            int dim, int vdim, int size, int pool, int page_size, int TQ, int S,
+                                            int Emax, float scale, hipStream_t stream) {
+  if (N <= 0) return 0;
+  if (H < 1 || G < 1 || H % G || H / G > kGroupMax || dim < 1 || vdim < 1 || vdim > kChanMax * kWave || size < 1 ||
+      pool < 1 || page_size < 1 || TQ < 1 || TQ > kTileMax || TQ * (H / G) > kPairMax || S < 1 || Emax < 1 ||
+      (long)KE * pool < (long)G * dim || (long)VE * pool < (long)G * vdim)
+    return -2;
+  SplitArgs a{positions, req_of_token, q_start, tables, talk, k_pool, v_pool, scores, part_m, part_l, part_o,
+              table_width, N, H, G, dim, vdim, size, pool, page_size, TQ, S, Emax, KE, VE, scale};
+  if (dtype == 0) return launch_split<float>(q, k_cache, v_cache, out, a, stream);
+  return launch_split<bf16_t>(q, k_cache, v_cache, out, a, stream);
+}
+
 TK_SLOTS(tk_bias_norm_store)
 TK_SLOTS(tk_pool_blocks)
 TK_SLOTS(tk_pooled_window_attention)
+TK_SLOTS(tk_pooled_window_attention_split)

@@ -7,7 +7,7 @@
 // wkv_scan: per (request, head) the recurrence
 //     o_t = (S + diag(u) k_t v_t^T)^T r_t ;  S <- diag(w_t) S + k_t v_t^T ,  w_t = exp(-exp(d_t + w0))
 //   over the step's tokens in order, the state S [dim, dim] in float32 registers (a thread owns a
-//   column), followed by the head's unit norm, a gain and a SiLU gate.
+//   few key channels of a column), followed by the head's unit norm, a gain and a SiLU gate.
 //
 // Decays, exponentials, the state and the norm are float32 whatever the storage type.
 #include "common.h"
@@ -33,20 +33,21 @@ __global__ void token_shift_kernel(const T* __restrict__ h, const float* __restr
                                    const int* __restrict__ req_of_token, const int* __restrict__ q_start,
                                    const int* __restrict__ state_slots, int N, int W, int S) {
   const int n = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;      // a thread a column: no loop whose loads wait for one another
+  if (c >= W) return;
   const int r = req_of_token[n];
   const int first = q_start[r];
   const int end = q_start[r + 1];
   const bool head = n == first;
   float* mine = last + (size_t)state_slots[r] * W;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    const float cur = Elem<T>::load(h + (size_t)n * W + c);
-    const float prev = head ? mine[c] : Elem<T>::load(h + (size_t)(n - 1) * W + c);
-    const float d = prev - cur;
-    for (int s = 0; s < S; ++s)
-      Elem<T>::store(out + ((size_t)s * N + n) * W + c, cur + d * mu[(size_t)s * W + c]);
-    // the thread that has read the old row of the state is the one that replaces it
-    if (head) mine[c] = Elem<T>::load(h + (size_t)(end - 1) * W + c);
-  }
+  const float cur = Elem<T>::load(h + (size_t)n * W + c);
+  const float prev = head ? mine[c] : Elem<T>::load(h + (size_t)(n - 1) * W + c);
+  const float newest = head ? Elem<T>::load(h + (size_t)(end - 1) * W + c) : 0.f;
+  const float d = prev - cur;
+  for (int s = 0; s < S; ++s)
+    Elem<T>::store(out + ((size_t)s * N + n) * W + c, cur + d * mu[(size_t)s * W + c]);
+  // the thread that has read the old row of the state is the one that replaces it
+  if (head) mine[c] = newest;
 }
 
 template <typename T>
@@ -59,47 +60,63 @@ __global__ void tanh_kernel(const void* __restrict__ in, int f32, int parts, lon
 
 constexpr int kScanTokens = 8;   // tokens whose operands are staged in LDS at once
 
-template <typename T, int DMAX>
-__global__ __launch_bounds__(DMAX < 64 ? 64 : DMAX) void wkv_scan_kernel(
+struct ScanShape {
+  int heads, dim, columns, slices, slice;   // threads = columns * slices; a thread owns `slice` key channels of a column
+};
+
+// A block a (request, head).  Thread (ks, j) owns the state's rows [ks * slice, (ks + 1) * slice)
+// of column j in registers: the key channels of a head are cut over `slices` groups of threads, so
+// that a token costs each thread `slice` multiply-adds and not `dim`; the groups' partial
+// outputs meet in LDS.  Tokens run in order, eight staged at a time.
+template <typename T, int SLICE>
+__global__ __launch_bounds__(1024) void wkv_scan_kernel(
     const T* __restrict__ r_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
     const T* __restrict__ g_in, const void* __restrict__ d_in, int d_f32, int d_parts, long d_stride,
     const float* __restrict__ w0, const float* __restrict__ u, const float* __restrict__ gain,
     float* __restrict__ state, const int* __restrict__ q_start, const int* __restrict__ state_slots,
-    T* __restrict__ out, int heads, int dim, float eps) {
+    T* __restrict__ out, ScanShape sh, float eps) {
   constexpr int TB = kScanTokens;
-  __shared__ float rr[TB][DMAX], kk[TB][DMAX], ww[TB][DMAX], uk[TB][DMAX], os[TB][DMAX];
-  __shared__ float rstd[TB];
+  extern __shared__ float lds[];
+  const int dim = sh.dim, CT = sh.columns, KS = sh.slices, slice = sh.slice;
+  const int dimp = (dim + 3) & ~3;
+  float* rr = lds;                     // [TB][dimp] each
+  float* kk = rr + TB * dimp;
+  float* ww = kk + TB * dimp;
+  float* uk = ww + TB * dimp;
+  float* os = uk + TB * dimp;
+  float* rstd = os + TB * dimp;        // [TB]
+  float* part = rstd + TB;             // [KS][TB][CT]
   const int req = blockIdx.x, head = blockIdx.y;
-  const int j = threadIdx.x;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int ks = tid / CT, j = tid - ks * CT;
   const bool live = j < dim;
-  const int HD = heads * dim;
-  const int col = head * dim + j;
+  const int k0 = ks * slice;
+  const int kn = max(0, min(slice, dim - k0));     // key channels of this thread's slice that exist
+  const int HD = sh.heads * dim;
+  const int base = head * dim;
   const int first = q_start[req], end = q_start[req + 1];
-  float* S = state + ((size_t)state_slots[req] * heads + head) * dim * dim;
-  float s[DMAX];
+  float* S = state + ((size_t)state_slots[req] * sh.heads + head) * dim * dim;
+  float s[SLICE];
 #pragma unroll
-  for (int x = 0; x < DMAX; ++x) s[x] = (live && x < dim) ? S[(size_t)x * dim + j] : 0.f;
-  const float w0j = live ? w0[col] : 0.f, uj = live ? u[col] : 0.f, gj = live ? gain[col] : 0.f;
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int nwaves = (blockDim.x + kWave - 1) / kWave;
+  for (int x = 0; x < SLICE; ++x) s[x] = (live && x < kn) ? S[(size_t)(k0 + x) * dim + j] : 0.f;
+  const float gj = live ? gain[base + j] : 0.f;
+  const int lane = tid & (kWave - 1), wave = tid / kWave, nwaves = nthreads / kWave;
 
   for (int t0 = first; t0 < end; t0 += TB) {
     const int tb = min(TB, end - t0);
-    float vloc[TB], gloc[TB];
-#pragma unroll
-    for (int t = 0; t < TB; ++t) {
-      vloc[t] = gloc[t] = 0.f;
-      if (t < tb && live) {
-        const size_t at = (size_t)(t0 + t) * HD + col;
-        const float kv = Elem<T>::load(k_in + at);
-        rr[t][j] = Elem<T>::load(r_in + at);
-        kk[t][j] = kv;
-        uk[t][j] = uj * kv;
-        ww[t][j] = expf(-expf(load_in<T>(d_in, d_f32, d_parts, d_stride, at) + w0j));
-        vloc[t] = Elem<T>::load(v_in + at);
-        gloc[t] = Elem<T>::load(g_in + at);
-      }
+    for (int i = tid; i < tb * dim; i += nthreads) {
+      const int t = i / dim, c = i - t * dim;
+      const size_t at = (size_t)(t0 + t) * HD + base + c;
+      const float kv = Elem<T>::load(k_in + at);
+      rr[t * dimp + c] = Elem<T>::load(r_in + at);
+      kk[t * dimp + c] = kv;
+      uk[t * dimp + c] = u[base + c] * kv;
+      ww[t * dimp + c] = expf(-expf(load_in<T>(d_in, d_f32, d_parts, d_stride, at) + w0[base + c]));
     }
+    float vloc[TB];
+#pragma unroll
+    for (int t = 0; t < TB; ++t)
+      vloc[t] = (t < tb && live) ? Elem<T>::load(v_in + (size_t)(t0 + t) * HD + base + j) : 0.f;
     __syncthreads();
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
@@ -107,38 +124,55 @@ __global__ __launch_bounds__(DMAX < 64 ? 64 : DMAX) void wkv_scan_kernel(
         const float vj = vloc[t];
         float o = 0.f;
 #pragma unroll
-        for (int x = 0; x < DMAX; ++x) {
-          if (x < dim) {
-            o = fmaf(rr[t][x], fmaf(uk[t][x], vj, s[x]), o);
-            s[x] = fmaf(ww[t][x], s[x], kk[t][x] * vj);
+        for (int x = 0; x < SLICE; x += 4) {
+          if (x < kn) {
+            const int at = t * dimp + k0 + x;       // (k0 and dimp are multiples of four)
+            const float4 r4 = *reinterpret_cast<const float4*>(rr + at);
+            const float4 k4 = *reinterpret_cast<const float4*>(kk + at);
+            const float4 w4 = *reinterpret_cast<const float4*>(ww + at);
+            const float4 u4 = *reinterpret_cast<const float4*>(uk + at);
+            const float rv[4] = {r4.x, r4.y, r4.z, r4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w};
+            const float wv[4] = {w4.x, w4.y, w4.z, w4.w}, uv[4] = {u4.x, u4.y, u4.z, u4.w};
+#pragma unroll
+            for (int y = 0; y < 4; ++y) {
+              if (x + y < kn) {
+                o = fmaf(rv[y], fmaf(uv[y], vj, s[x + y]), o);
+                s[x + y] = fmaf(wv[y], s[x + y], kv[y] * vj);
+              }
+            }
           }
         }
-        if (live) os[t][j] = o;
+        part[(ks * TB + t) * CT + j] = o;
       }
+    }
+    __syncthreads();
+    for (int t = ks; t < tb; t += KS) {
+      float o = 0.f;
+      for (int q = 0; q < KS; ++q) o += part[(q * TB + t) * CT + j];
+      if (live) os[t * dimp + j] = o;
     }
     __syncthreads();
     for (int t = wave; t < tb; t += nwaves) {
       float q = 0.f;
-      for (int x = lane; x < dim; x += kWave) q += os[t][x] * os[t][x];
+      for (int x = lane; x < dim; x += kWave) q += os[t * dimp + x] * os[t * dimp + x];
       q = wave_sum(q);
       if (lane == 0) rstd[t] = 1.f / sqrtf(q / (float)dim + eps);
     }
     __syncthreads();
-#pragma unroll
-    for (int t = 0; t < TB; ++t) {
-      if (t < tb && live) {
-        const float g = gloc[t];
-        const float y = os[t][j] * rstd[t] * gj * (g / (1.f + expf(-g)));
-        Elem<T>::store(out + (size_t)(t0 + t) * HD + col, y);
+    for (int t = ks; t < tb; t += KS) {
+      if (live) {
+        const size_t at = (size_t)(t0 + t) * HD + base + j;
+        const float g = Elem<T>::load(g_in + at);
+        Elem<T>::store(out + at, os[t * dimp + j] * rstd[t] * gj * (g / (1.f + expf(-g))));
       }
     }
-    // (the next round writes rr, kk, ww, uk, which nobody reads after the second barrier, and
-    // os and rstd only behind its own barriers)
+    // (the next round's staging writes rr, kk, ww, uk, which nobody reads after the second
+    // barrier; os, rstd and part are written again only behind the next round's barriers)
   }
   if (live) {
 #pragma unroll
-    for (int x = 0; x < DMAX; ++x)
-      if (x < dim) S[(size_t)x * dim + j] = s[x];
+    for (int x = 0; x < SLICE; ++x)
+      if (x < kn) S[(size_t)(k0 + x) * dim + j] = s[x];
   }
 }
 
@@ -147,15 +181,33 @@ int launch_scan(const void* r, const void* k, const void* v, const void* g, cons
                 long d_stride, const float* w0, const float* u, const float* gain, float* state,
                 const int* q_start, const int* state_slots, void* out, int R, int heads, int dim, float eps,
                 hipStream_t stream) {
+  ScanShape sh;
+  sh.heads = heads;
+  sh.dim = dim;
+  sh.columns = (dim + kWave - 1) / kWave * kWave;
+  const int most = min(16, 1024 / sh.columns);                      // groups of threads that can share a head
+  sh.slice = max(4, ((dim + most - 1) / most + 3) / 4 * 4);
+  sh.slices = (dim + sh.slice - 1) / sh.slice;
+  const int threads = sh.columns * sh.slices;
+  const int dimp = (dim + 3) & ~3;
+  const size_t lds = ((size_t)5 * kScanTokens * dimp + kScanTokens + (size_t)sh.slices * kScanTokens * sh.columns) * 4;
   const dim3 grid(R, heads);
-#define TK_SCAN(DMAX)                                                                                    \
-  wkv_scan_kernel<T, DMAX><<<grid, (DMAX < 64 ? 64 : DMAX), 0, stream>>>(                                 \
-      (const T*)r, (const T*)k, (const T*)v, (const T*)g, d, d_f32, d_parts, d_stride, w0, u, gain, state, \
-      q_start, state_slots, (T*)out, heads, dim, eps)
-  if (dim <= 32) TK_SCAN(32);
-  else if (dim <= 64) TK_SCAN(64);
-  else if (dim <= 128) TK_SCAN(128);
-  else TK_SCAN(256);
+#define TK_SCAN(SLICE)                                                                                        \
+  {                                                                                                           \
+    static bool allowed = false;                                                                              \
+    if (!allowed) {                                                                                           \
+      const hipError_t err = hipFuncSetAttribute((const void*)wkv_scan_kernel<T, SLICE>,                      \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);     \
+      if (err != hipSuccess) return (int)err;                                                                 \
+      allowed = true;                                                                                         \
+    }                                                                                                         \
+    wkv_scan_kernel<T, SLICE><<<grid, threads, lds, stream>>>(                                                \
+        (const T*)r, (const T*)k, (const T*)v, (const T*)g, d, d_f32, d_parts, d_stride, w0, u, gain, state,  \
+        q_start, state_slots, (T*)out, sh, eps);                                                              \
+  }
+  if (sh.slice <= 4) TK_SCAN(4)
+  else if (sh.slice <= 16) TK_SCAN(16)
+  else TK_SCAN(64)
 #undef TK_SCAN
   return launch_status();
 }
@@ -168,12 +220,13 @@ TK_API int tk_token_shift(int dtype, const void* h, const float* mu, float* last
                           const int* req_of_token, const int* q_start, const int* state_slots, int N, int W,
                           int S, hipStream_t stream) {
   if (N <= 0 || W <= 0 || S <= 0) return 0;
-  const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+  const int threads = W >= 256 ? 256 : 64;
+  const dim3 grid(N, (W + threads - 1) / threads);
   if (dtype == 0)
-    token_shift_kernel<float><<<N, threads, 0, stream>>>((const float*)h, mu, last, (float*)out, req_of_token,
+    token_shift_kernel<float><<<grid, threads, 0, stream>>>((const float*)h, mu, last, (float*)out, req_of_token,
                                                          q_start, state_slots, N, W, S);
   else
-    token_shift_kernel<bf16_t><<<N, threads, 0, stream>>>((const bf16_t*)h, mu, last, (bf16_t*)out, req_of_token,
+    token_shift_kernel<bf16_t><<<grid, threads, 0, stream>>>((const bf16_t*)h, mu, last, (bf16_t*)out, req_of_token,
                                                           q_start, state_slots, N, W, S);
   return launch_status();
 }

@@ -91,6 +91,24 @@ class AttentionWork(StepPlanner):
 ATTENTION_WORK = AttentionWork()
 
 
+class ContextLength(StepPlanner):
+    """The longest context of a step (cached tokens plus the step's own) as a fact, for kernels
+    that size scratch memory and grids by the entries a row can see.  Recorded steps round it up,
+    four values an octave: a recording then serves every step up to the rounded length."""
+
+    name = "context"
+
+    def lists(self, q_lens, ctx_lens):
+        return {}, {"max_len": max((c + q for q, c in zip(q_lens, ctx_lens)), default=0)}
+
+    def bucket(self, facts):
+        facts["max_len"] = quarter_octave_at_least(facts["max_len"], 64)
+        return facts
+
+
+CONTEXT_LENGTH = ContextLength()
+
+
 class _Work:
     """The attention planner's lists and facts of a step, by attribute."""
 

@@ -189,6 +189,12 @@ _SIGS = {
                                        c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_float, c_void_p],
     },
+    "attention_pooled_split": {
+        "tk_pooled_window_attention_split": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                             c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                             c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    },
     "recurrent": {
         "tk_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                            c_int, c_int, c_void_p],
@@ -247,7 +253,7 @@ _SIGS = {
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     },
 }
-_LIBRARY_FILE = {"attention_fused": "attention_mfma"}   # signature group -> library that holds it
+_LIBRARY_FILE = {"attention_fused": "attention_mfma", "attention_pooled_split": "attention_pooled"}   # signature group -> library that holds it
 _fns: dict[str, ctypes._CFuncPtr] = {}
 _profile: "KernelProfile | None" = None
 
@@ -562,6 +568,34 @@ def pooled_window_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, l
     return rows, chunk, threads
 
 
+POOLED_SPLIT_GROUP = 16      # query heads a kv head, value channels and rows times heads a block
+POOLED_SPLIT_VDIM = 256      # that the three-kernel form of the attention takes
+POOLED_SPLIT_PAIRS = 32
+POOLED_SPLIT_BLOCKS = 1024   # blocks wanted in flight
+POOLED_SPLIT_LDS = 150 * 1024
+
+
+def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, window: int, pool: int, n: int,
+                      longest_span: int, longest_context: int) -> tuple[int, int, int] | None:
+    """(rows a block, shares of the entries, most entries a tile sees) for the three-kernel form of
+    the pooled-window attention, or None where its sizes do not fit and the one-kernel form runs.
+    Up to 8 consecutive rows of a portion share the rows a lane loads; single tokens take a
+    block each; the entries are cut in shares until about a thousand blocks exist."""
+    group = num_heads // num_kv_heads
+    if group > POOLED_SPLIT_GROUP or vdim > POOLED_SPLIT_VDIM:
+        return None
+    rows = 1 if longest_span <= 1 else max(1, min(8, POOLED_SPLIT_PAIRS // group))
+    while rows > 1 and 4 * (2 * rows * num_heads + group * num_heads + rows * group * (256 + 4 * vdim)) > POOLED_SPLIT_LDS:
+        rows //= 2
+    if (4 * (2 * rows * num_heads + group * num_heads + rows * group * (256 + 4 * vdim)) > POOLED_SPLIT_LDS
+            or 4 * (rows * group * dim + 8 * POOLED_SPLIT_PAIRS) > POOLED_SPLIT_LDS):
+        return None
+    most = min(longest_context, window + rows - 1) + longest_context // pool + 1
+    blocks = -(-n // rows) * num_kv_heads
+    shares = max(1, min(32, -(-POOLED_SPLIT_BLOCKS // blocks), -(-most // 128)))
+    return rows, shares, most
+
+
 def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, k_pool: torch.Tensor,
                             v_pool: torch.Tensor, tables: torch.Tensor, batch, talk: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                             dim: int, vdim: int, window: int, pool: int, page_size: int, scale: float) -> None:
@@ -581,7 +615,6 @@ def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _need(batch.num_tokens == n and tables.shape[0] == batch.num_requests and tables.dtype == torch.int32,
           "block tables do not match the step")
     _need(-(-batch.max_seq_len // page_size) <= tables.shape[1], "a block table is shorter than its request")
-    rows, chunk, threads = pooled_window_plan(num_heads, num_kv_heads, dim, vdim, batch.max_q_len)
     if _profile is not None:
         # the least a step has to move: every cached position of every request once, queries in,
         # results out; and two multiply-adds per head, channel and visible entry
@@ -594,6 +627,23 @@ def pooled_window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         cached = sum(min(c + ql, window + ql - 1) * elem + (c + ql) // pool * 4 for c, ql in zip(batch.ctx_lens, batch.q_lens))
         _note(f"{n}x{num_heads}x{dim}", cached * num_kv_heads * (dim + vdim) + n * num_heads * (dim + vdim) * elem,
               2.0 * num_heads * (dim + vdim) * entries)
+    split = pooled_split_plan(num_heads, num_kv_heads, dim, vdim, window, pool, n, batch.max_q_len,
+                              batch.facts.get("context.max_len", batch.max_seq_len))
+    if split is not None:
+        # the form that fills the GPU: a block a (tile of rows, kv head, share of the entries)
+        rows, shares, most = split
+        dev = q.device
+        scores = torch.empty((n, most, num_heads), dtype=torch.float32, device=dev)
+        part_m = torch.empty((n, num_heads, shares), dtype=torch.float32, device=dev)
+        part_l = torch.empty((n, num_heads, shares), dtype=torch.float32, device=dev)
+        part_o = torch.empty((shares, n, num_heads * vdim), dtype=torch.float32, device=dev) if shares > 1 else None
+        _check(_fn("attention_pooled_split", "tk_pooled_window_attention_split")(
+            _code(dtype), _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool), ke, ve, _p(out), _p(batch.positions),
+            _p(batch.req_of_token), _p(batch.q_start), _p(tables), tables.shape[1], _p(talk), _p(scores), _p(part_m),
+            _p(part_l), _p(part_o), n, num_heads, num_kv_heads, dim, vdim, window, pool, page_size, rows, shares, most,
+            float(scale), _stream()), "pooled_window_attention_split")
+        return
+    rows, chunk, threads = pooled_window_plan(num_heads, num_kv_heads, dim, vdim, batch.max_q_len)
     _check(_fn("attention_pooled", "tk_pooled_window_attention")(
         _code(dtype), _p(q), _p(k_cache), _p(v_cache), _p(k_pool), _p(v_pool), ke, ve, _p(out), _p(batch.positions),
         _p(batch.req_of_token), _p(batch.q_start), _p(tables), tables.shape[1], _p(talk), n, num_heads, num_kv_heads, dim, vdim, window, pool,

@@ -6,6 +6,7 @@ import torch
 
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
+from tokamak_amd.kernels.attention import CONTEXT_LENGTH
 from tokamak_amd.kernels.linear import linear
 from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer, PagedArray, PositionData
 from tokamak_amd.weights.spec import TensorSpec
@@ -79,6 +80,9 @@ class PooledWindowAttention(Mixer):
         return CacheRequest.of(window=None, k=self.k_width, v=self.v_width,
                                k_pool=PagedArray(ops.pooled_elems(self.k_width, self.pool), torch.float32),
                                v_pool=PagedArray(ops.pooled_elems(self.v_width, self.pool), torch.float32))
+
+    def step_planner(self):
+        return CONTEXT_LENGTH
 
     def pair_flops(self) -> float:
         return 2.0 * self.num_heads * (self.head_dim + self.value_dim)
