@@ -113,6 +113,66 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(
   }
 }
 
+// The same for rows of up to 8 * 1024 numbers: a thread holds its eight in registers, so every
+// load of the row is asked for at once and the row is read once.
+constexpr int kRowRegs = 8;
+template <typename T>
+__global__ __launch_bounds__(1024) void bias_norm_store_row_kernel(
+    const void* __restrict__ qkv, int in_f32, int parts, long part_stride, const float* __restrict__ bias,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, const int* __restrict__ positions,
+    const int* __restrict__ req_of_token, const int* __restrict__ tables, int table_width,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int QW, int KW, int VW,
+    int page_size, float eps, int store) {
+  __shared__ float scratch[16];
+  const int n = blockIdx.x;
+  const int total = store ? QW + KW + VW : QW;
+  const size_t row = (size_t)n * total;
+  float x[kRowRegs];
+#pragma unroll
+  for (int u = 0; u < kRowRegs; ++u) {
+    const int c = threadIdx.x + u * blockDim.x;
+    x[u] = c < total ? bias[c] : 0.f;
+  }
+  if (!in_f32) {
+#pragma unroll
+    for (int u = 0; u < kRowRegs; ++u) {
+      const int c = threadIdx.x + u * blockDim.x;
+      if (c < total) x[u] += Elem<T>::load(reinterpret_cast<const T*>(qkv) + row + c);
+    }
+  } else {
+    const float* f = reinterpret_cast<const float*>(qkv);
+    for (int i = 0; i < parts; ++i) {
+#pragma unroll
+      for (int u = 0; u < kRowRegs; ++u) {
+        const int c = threadIdx.x + u * blockDim.x;
+        if (c < total) x[u] += f[row + c + (size_t)i * part_stride];
+      }
+    }
+  }
+  float sq = 0.f, sk = 0.f;
+#pragma unroll
+  for (int u = 0; u < kRowRegs; ++u) {
+    const int c = threadIdx.x + u * blockDim.x;
+    if (c < QW) sq += x[u] * x[u];
+    else if (c < QW + KW) sk += x[u] * x[u];
+  }
+  sq = block_sum(sq, scratch);
+  if (store) sk = block_sum(sk, scratch);
+  const float rq = 1.f / sqrtf(sq / (float)QW + eps), rk = 1.f / sqrtf(sk / (float)KW + eps);
+  size_t slot = 0;
+  if (store) {
+    const int pos = positions[n];
+    slot = (size_t)tables[(size_t)req_of_token[n] * table_width + pos / page_size] * page_size + pos % page_size;
+  }
+#pragma unroll
+  for (int u = 0; u < kRowRegs; ++u) {
+    const int c = threadIdx.x + u * blockDim.x;
+    if (c < QW) Elem<T>::store(q_out + (size_t)n * QW + c, x[u] * rq * q_weight[c]);
+    else if (c < QW + KW) Elem<T>::store(k_cache + slot * KW + (c - QW), x[u] * rk * k_weight[c - QW]);
+    else if (c < total) Elem<T>::store(v_cache + slot * VW + (c - QW - KW), x[u]);
+  }
+}
+
 struct PoolArgs {
   const int* positions;
   const int* req_of_token;
@@ -402,30 +462,39 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_scores_kernel(const T* _
         const int p = g.j0 + entry - g.NB;
         rowp = k_cache + ((size_t)g.table[p / a.page_size] * a.page_size + p % a.page_size) * KW + (size_t)c * dim;
       }
-      for (int x0 = 0; x0 < dim; x0 += 8) {
-        float kx[8];
-        if (rowp != nullptr && vec) {
-          load8(rowp + x0, kx);
-        } else if (poolp != nullptr && pvec) {
-          load8(poolp + x0, kx);
-        } else {
+      if ((rowp != nullptr && vec) || (poolp != nullptr && pvec)) {
+        // 64 elements of the row asked for at once (eight 16- or 32-byte loads in flight), then
+        // the products, the queries read from LDS four at a time
+        for (int x0 = 0; x0 < dim; x0 += 64) {
+          float kx[64];
 #pragma unroll
           for (int u = 0; u < 8; ++u) {
-            const int x = x0 + u;
-            kx[u] = x >= dim ? 0.f
-                    : rowp != nullptr ? Elem<T>::load(rowp + x)
-                    : poolp != nullptr ? poolp[x]
-                                       : entry_value<T>(k_cache, a.k_pool, g, entry, c * dim + x, KW, a.KE, a.page_size);
+            if (x0 + 8 * u < dim) {
+              if (rowp != nullptr) load8(rowp + x0 + 8 * u, kx + 8 * u);
+              else load8(poolp + x0 + 8 * u, kx + 8 * u);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 16; ++u) {
+            if (x0 + 4 * u < dim) {
+#pragma unroll
+              for (int p = 0; p < kPairMax; ++p) {
+                if (p < pairs) {
+                  const float4 qv = *reinterpret_cast<const float4*>(qs + p * dim + x0 + 4 * u);
+                  acc[p] = fmaf(qv.x, kx[4 * u], fmaf(qv.y, kx[4 * u + 1], fmaf(qv.z, kx[4 * u + 2], fmaf(qv.w, kx[4 * u + 3], acc[p]))));
+                }
+              }
+            }
           }
         }
-        const int left = min(8, dim - x0);
+      } else {
+        for (int x = 0; x < dim; ++x) {
+          const float kx = rowp != nullptr ? Elem<T>::load(rowp + x)
+                           : poolp != nullptr ? poolp[x]
+                                              : entry_value<T>(k_cache, a.k_pool, g, entry, c * dim + x, KW, a.KE, a.page_size);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          if (u < left) {
-#pragma unroll
-            for (int p = 0; p < kPairMax; ++p)
-              if (p < pairs) acc[p] = fmaf(qs[p * dim + x0 + u], kx[u], acc[p]);
-          }
+          for (int p = 0; p < kPairMax; ++p)
+            if (p < pairs) acc[p] = fmaf(qs[p * dim + x], kx, acc[p]);
         }
       }
 #pragma unroll
@@ -493,17 +562,27 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
     const Segment g = segment_at(a, row, row_end);
     const int pairs = g.tq * group;
     __syncthreads();
-    for (int i = tid; i < g.tq * H; i += kSplitThreads) {
-      const size_t at = ((size_t)(g.row + i / H) * H + i % H) * a.S;
-      float m_all = -INFINITY;
-      for (int s = 0; s < a.S; ++s) m_all = fmaxf(m_all, a.part_m[at + s]);
-      float l_all = 0.f;
-      for (int s = 0; s < a.S; ++s) {
-        const float ms = a.part_m[at + s];
-        if (ms > -INFINITY) l_all += a.part_l[at + s] * expf(ms - m_all);
+    // the shares' statistics of every (row, head): loaded side by side, merged from LDS
+    {
+      float* sm_ = wm;                                 // [tq * H][S] maxima, then as many sums
+      const int count = g.tq * H * a.S;
+      const size_t from = (size_t)g.row * H * a.S;     // (the rows of a segment follow one another)
+      for (int i = tid; i < count; i += kSplitThreads) {
+        sm_[i] = a.part_m[from + i];
+        sm_[count + i] = a.part_l[from + i];
       }
-      mh[i] = m_all;
-      il[i] = 1.f / l_all;
+      __syncthreads();
+      for (int i = tid; i < g.tq * H; i += kSplitThreads) {
+        float m_all = -INFINITY;
+        for (int sh = 0; sh < a.S; ++sh) m_all = fmaxf(m_all, sm_[i * a.S + sh]);
+        float l_all = 0.f;
+        for (int sh = 0; sh < a.S; ++sh) {
+          const float ms = sm_[i * a.S + sh];
+          if (ms > -INFINITY) l_all += sm_[count + i * a.S + sh] * expf(ms - m_all);
+        }
+        mh[i] = m_all;
+        il[i] = 1.f / l_all;
+      }
     }
     __syncthreads();
     const int e_lo = (int)((long)g.E * split / a.S), e_hi = (int)((long)g.E * (split + 1) / a.S);
@@ -521,12 +600,41 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
           float mixed[kGroupMax];
 #pragma unroll
           for (int h = 0; h < kGroupMax; ++h) mixed[h] = 0.f;
-          for (int gh = 0; gh < H; ++gh) {
-            const float s = sc[gh];
-            const float w = s > -INFINITY ? expf(s - mh[t * H + gh]) * il[t * H + gh] : 0.f;
+          if (H % 4 == 0) {
+            float4 ahead[8];        // the scores of 32 heads asked for at once
 #pragma unroll
-            for (int h = 0; h < kGroupMax; ++h)
-              if (h < group) mixed[h] = fmaf(tk_[h * H + gh], w, mixed[h]);
+            for (int y = 0; y < 8; ++y)
+              if (4 * y < H) ahead[y] = *reinterpret_cast<const float4*>(sc + 4 * y);
+            for (int gh = 0; gh < H; gh += 4) {
+              float4 s4;
+              if (gh < 32) {
+#pragma unroll
+                for (int y = 0; y < 8; ++y)
+                  if (gh == 4 * y) s4 = ahead[y];
+              } else {
+                s4 = *reinterpret_cast<const float4*>(sc + gh);
+              }
+              const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
+              float w[4];
+#pragma unroll
+              for (int y = 0; y < 4; ++y)
+                w[y] = sv[y] > -INFINITY ? expf(sv[y] - mh[t * H + gh + y]) * il[t * H + gh + y] : 0.f;
+#pragma unroll
+              for (int h = 0; h < kGroupMax; ++h) {
+                if (h < group) {
+                  const float4 t4 = *reinterpret_cast<const float4*>(tk_ + h * H + gh);
+                  mixed[h] = fmaf(t4.x, w[0], fmaf(t4.y, w[1], fmaf(t4.z, w[2], fmaf(t4.w, w[3], mixed[h]))));
+                }
+              }
+            }
+          } else {
+            for (int gh = 0; gh < H; ++gh) {
+              const float s = sc[gh];
+              const float w = s > -INFINITY ? expf(s - mh[t * H + gh]) * il[t * H + gh] : 0.f;
+#pragma unroll
+              for (int h = 0; h < kGroupMax; ++h)
+                if (h < group) mixed[h] = fmaf(tk_[h * H + gh], w, mixed[h]);
+            }
           }
 #pragma unroll
           for (int h = 0; h < kGroupMax; ++h)
@@ -534,19 +642,30 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
         }
       }
       __syncthreads();
-      for (int e = wave; e < ne; e += kWaves) {
-        float v[kChanMax];
+      for (int e = wave; e < ne; e += 4 * kWaves) {      // four entries' values asked for at once
+        float v[4][kChanMax];
 #pragma unroll
-        for (int d = 0; d < kChanMax; ++d) {
-          const int x = lane + d * kWave;
-          v[d] = x < vdim ? entry_value<T>(v_cache, a.v_pool, g, e0 + e, c * vdim + x, VW, a.VE, a.page_size) : 0.f;
+        for (int y = 0; y < 4; ++y) {
+          const int ee = e + y * kWaves;
+#pragma unroll
+          for (int d = 0; d < kChanMax; ++d) {
+            const int x = lane + d * kWave;
+            v[y][d] = (ee < ne && x < vdim)
+                          ? entry_value<T>(v_cache, a.v_pool, g, e0 + ee, c * vdim + x, VW, a.VE, a.page_size) : 0.f;
+          }
         }
 #pragma unroll
-        for (int p = 0; p < kPairMax; ++p) {
-          if (p < pairs) {
-            const float w = wm[p * kSplitThreads + e];
+        for (int y = 0; y < 4; ++y) {
+          const int ee = e + y * kWaves;
+          if (ee < ne) {
 #pragma unroll
-            for (int d = 0; d < kChanMax; ++d) acc[p][d] = fmaf(w, v[d], acc[p][d]);
+            for (int p = 0; p < kPairMax; ++p) {
+              if (p < pairs) {
+                const float w = wm[p * kSplitThreads + ee];
+#pragma unroll
+                for (int d = 0; d < kChanMax; ++d) acc[p][d] = fmaf(w, v[y][d], acc[p][d]);
+              }
+            }
           }
         }
       }
@@ -591,8 +710,10 @@ int launch_split(const void* q, const void* k_cache, const void* v_cache, void* 
   const int group = a.H / a.G;
   const dim3 grid((a.N + a.TQ - 1) / a.TQ, a.G, a.S);
   const size_t lds_a = ((size_t)a.TQ * group * a.dim + (kSplitThreads / kWave) * kPairMax * 2) * 4;
-  const size_t lds_b = ((size_t)2 * a.TQ * a.H + (size_t)group * a.H + (size_t)a.TQ * group * kSplitThreads +
-                        (size_t)(kSplitThreads / kWave) * a.TQ * group * a.vdim) * 4;
+  // (the shares' statistics are merged in the space of the mixed weights and the waves' sums)
+  const size_t work = (size_t)a.TQ * group * kSplitThreads + (size_t)(kSplitThreads / kWave) * a.TQ * group * a.vdim;
+  const size_t stats = (size_t)2 * a.TQ * a.H * a.S;
+  const size_t lds_b = ((size_t)2 * a.TQ * a.H + (size_t)group * a.H + (work > stats ? work : stats)) * 4;
   if (lds_a > 150 * 1024 || lds_b > 150 * 1024) return -3;
   static bool allowed = false;      // (per instantiation: once per storage type)
   if (!allowed) {
@@ -623,6 +744,19 @@ TK_API int tk_bias_norm_store(int dtype, const void* qkv, int in_f32, int parts,
                               int page_size, float eps, int store, hipStream_t stream) {
   if (N <= 0) return 0;
   if (QW < 1 || KW < 1 || VW < 1 || page_size < 1) return -2;
+  const int total = store ? QW + KW + VW : QW;
+  if (total <= kRowRegs * 1024) {
+    const int threads = total >= 4096 ? 1024 : (total >= 1024 ? 512 : 256);
+    if (dtype == 0)
+      bias_norm_store_row_kernel<float><<<N, threads, 0, stream>>>(
+          qkv, in_f32, parts, part_stride, bias, q_weight, k_weight, positions, req_of_token, tables, table_width,
+          (float*)q_out, (float*)k_cache, (float*)v_cache, QW, KW, VW, page_size, eps, store);
+    else
+      bias_norm_store_row_kernel<bf16_t><<<N, threads, 0, stream>>>(
+          qkv, in_f32, parts, part_stride, bias, q_weight, k_weight, positions, req_of_token, tables, table_width,
+          (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, QW, KW, VW, page_size, eps, store);
+    return launch_status();
+  }
   if (dtype == 0)
     bias_norm_store_kernel<float><<<N, 256, 0, stream>>>(qkv, in_f32, parts, part_stride, bias, q_weight, k_weight,
                                                          positions, req_of_token, tables, table_width, (float*)q_out,

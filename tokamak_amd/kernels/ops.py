@@ -571,7 +571,7 @@ def pooled_window_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, l
 POOLED_SPLIT_GROUP = 16      # query heads a kv head, value channels and rows times heads a block
 POOLED_SPLIT_VDIM = 256      # that the three-kernel form of the attention takes
 POOLED_SPLIT_PAIRS = 32
-POOLED_SPLIT_BLOCKS = 1024   # blocks wanted in flight
+POOLED_SPLIT_BLOCKS = 512    # blocks wanted: two a CU run at once (some 200 registers a lane), a third waits for a whole turn
 POOLED_SPLIT_LDS = 150 * 1024
 
 
@@ -581,18 +581,26 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
     the pooled-window attention, or None where its sizes do not fit and the one-kernel form runs.
     Up to 8 consecutive rows of a portion share the rows a lane loads; single tokens take a
     block each; the entries are cut in shares until about a thousand blocks exist."""
+    from tokamak_amd.kernels.attention import quarter_octave_at_least
+
     group = num_heads // num_kv_heads
     if group > POOLED_SPLIT_GROUP or vdim > POOLED_SPLIT_VDIM:
         return None
+    # the length rounded as recorded steps round it: a step computes the same bits recorded or not
+    longest_context = quarter_octave_at_least(longest_context, 64)
     rows = 1 if longest_span <= 1 else max(1, min(8, POOLED_SPLIT_PAIRS // group))
-    while rows > 1 and 4 * (2 * rows * num_heads + group * num_heads + rows * group * (256 + 4 * vdim)) > POOLED_SPLIT_LDS:
+    def values_lds(rows: int) -> int:       # (the statistics of up to 4,096 (row, head, share) triples are merged in the work space)
+        return 4 * (2 * rows * num_heads + group * num_heads + max(rows * group * (256 + 4 * vdim), 2 * 4096))
+
+    while rows > 1 and values_lds(rows) > POOLED_SPLIT_LDS:
         rows //= 2
-    if (4 * (2 * rows * num_heads + group * num_heads + rows * group * (256 + 4 * vdim)) > POOLED_SPLIT_LDS
-            or 4 * (rows * group * dim + 8 * POOLED_SPLIT_PAIRS) > POOLED_SPLIT_LDS):
+    if (values_lds(rows) > POOLED_SPLIT_LDS or 4 * (rows * group * dim + 8 * POOLED_SPLIT_PAIRS) > POOLED_SPLIT_LDS
+            or rows * num_heads > 4096):
         return None
     most = min(longest_context, window + rows - 1) + longest_context // pool + 1
     blocks = -(-n // rows) * num_kv_heads
-    shares = max(1, min(32, -(-POOLED_SPLIT_BLOCKS // blocks), -(-most // 128)))
+    # (a share of at least 32 entries; the shares' statistics of a tile's rows and heads fit the LDS they are merged in)
+    shares = max(1, min(32, POOLED_SPLIT_BLOCKS // blocks, -(-most // 32), 4096 // (rows * num_heads)))
     return rows, shares, most
 
 
