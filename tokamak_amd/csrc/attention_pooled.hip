@@ -342,12 +342,12 @@ __global__ void pooled_window_attention_kernel(const T* __restrict__ q, const T*
 //            maximum and sum of exponentials over the share.
 //   values:  merges the shares' statistics of ALL heads, turns the scores of its entries into
 //            normalised weights, mixes them for its own query heads, and applies them to its
-//            kv head's values (a wave an entry, a lane a channel); float32 partial outputs.
+//            kv head's values (64 entries staged in LDS at a time; a thread owns four channels of a few
+//            (row, head) pairs); float32 partial outputs.
 //   merge:   adds the shares' partial outputs.
 constexpr int kGroupMax = 16;   // query heads a kv head
 constexpr int kTileMax = 8;     // rows a block
 constexpr int kPairMax = 32;    // rows times query heads a lane accumulates in the score kernel
-constexpr int kChanMax = 4;     // value channels a lane: vdim <= 256
 constexpr int kSplitThreads = 256;
 
 struct SplitArgs {
@@ -542,19 +542,58 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_scores_kernel(const T* _
   }
 }
 
+constexpr int kStage = 64;     // entries whose values are staged in LDS at once
+constexpr int kOwnMax = 8;     // (row, head) pairs a thread of the value kernel owns
+
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                     __uint_as_float(v.y & 0xffff0000u));
+}
+
+// four channels from column `col` on (the first `valid` exist) of an entry's value row
+template <typename T>
+__device__ __forceinline__ float4 load_unit(const T* __restrict__ cache, const float* __restrict__ pooled,
+                                            const Segment& g, int entry, int col, int valid, int width, int E,
+                                            int page_size, bool vec, bool pvec) {
+  if (entry < g.NB) {
+    if (pvec) {   // (a piece of four never crosses a page: rows and pages are multiples of four numbers)
+      const size_t flat = (size_t)entry * width + col, per_page = (size_t)page_size * E;
+      return load4(pooled + (size_t)g.table[flat / per_page] * per_page + flat % per_page);
+    }
+  } else if (vec) {
+    const int p = g.j0 + entry - g.NB;
+    return load4(cache + ((size_t)g.table[p / page_size] * page_size + p % page_size) * width + col);
+  }
+  float v[4];
+#pragma unroll
+  for (int y = 0; y < 4; ++y)
+    v[y] = y < valid ? entry_value<T>(cache, pooled, g, entry, col + y, width, E, page_size) : 0.f;
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+
 template <typename T>
 __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* __restrict__ v_cache,
                                                                       T* __restrict__ out, SplitArgs a) {
   extern __shared__ float lds[];
   const int H = a.H, group = a.H / a.G, vdim = a.vdim, VW = a.G * a.vdim;
   const int c = blockIdx.y, split = blockIdx.z;
-  constexpr int kWaves = kSplitThreads / kWave;
   float* mh = lds;                                   // [TQ][H]  maximum of every head
   float* il = mh + a.TQ * H;                         // [TQ][H]  1 / sum
   float* tk_ = il + a.TQ * H;                        // [group][H]
   float* wm = tk_ + group * H;                       // [TQ * group][kSplitThreads] mixed weights of a chunk
-  float* red = wm + a.TQ * group * kSplitThreads;    // [waves][TQ * group][vdim]
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int vdimp = (vdim + 3) & ~3, upr = vdimp / 4;   // a row padded to pieces of four channels
+  float* Vs = wm + a.TQ * group * kSplitThreads;     // [kStage][vdimp] values of a stage
+  const int tid = threadIdx.x;
+  // thread (pg, cg): channels [4 cg, 4 cg + 4) of the pairs [pg PP, (pg + 1) PP)
+  int CG = 1;
+  while (CG < upr) CG *= 2;
+  const int PG = kSplitThreads / CG, PP = (a.TQ * group + PG - 1) / PG;
+  const int cg = tid & (CG - 1), pg = tid / CG;
+  const bool owner = 4 * cg < vdim;
+  const bool vvec = vdim % 4 == 0;
+  const bool pvvec = vvec && ((long)a.page_size * a.VE) % 4 == 0;
   for (int i = tid; i < group * H; i += kSplitThreads) tk_[i] = a.talk[(size_t)(c * group + i / H) * H + i % H];
   const int row_end = min(a.N, (int)(blockIdx.x + 1) * a.TQ);
   int row = blockIdx.x * a.TQ;
@@ -586,11 +625,11 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
     }
     __syncthreads();
     const int e_lo = (int)((long)g.E * split / a.S), e_hi = (int)((long)g.E * (split + 1) / a.S);
-    float acc[kPairMax][kChanMax];
+    float acc[kOwnMax][4];
 #pragma unroll
-    for (int p = 0; p < kPairMax; ++p)
+    for (int p = 0; p < kOwnMax; ++p)
 #pragma unroll
-      for (int d = 0; d < kChanMax; ++d) acc[p][d] = 0.f;
+      for (int d = 0; d < 4; ++d) acc[p][d] = 0.f;
     for (int e0 = e_lo; e0 < e_hi; e0 += kSplitThreads) {
       const int ne = min(kSplitThreads, e_hi - e0);
       __syncthreads();            // the chunk before is applied
@@ -642,54 +681,68 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
         }
       }
       __syncthreads();
-      for (int e = wave; e < ne; e += 4 * kWaves) {      // four entries' values asked for at once
-        float v[4][kChanMax];
+      // the chunk's values 64 entries at a time through LDS (every thread asks for four pieces of
+      // four channels at once), then applied: a thread owns four channels of up to eight (row, head) pairs
+      for (int sub = 0; sub < ne; sub += kStage) {
+        const int nsub = min(kStage, ne - sub);
+        const int units = nsub * upr;
+        for (int i0 = tid; i0 < units; i0 += 4 * kSplitThreads) {
+          float4 val[4];
 #pragma unroll
-        for (int y = 0; y < 4; ++y) {
-          const int ee = e + y * kWaves;
+          for (int y = 0; y < 4; ++y) {
+            const int i = i0 + y * kSplitThreads;
+            if (i < units) {
+              const int e = i / upr, x = 4 * (i - e * upr);
+              val[y] = load_unit<T>(v_cache, a.v_pool, g, e0 + sub + e, c * vdim + x, vdim - x, VW, a.VE, a.page_size,
+                                    vvec, pvvec);
+            }
+          }
 #pragma unroll
-          for (int d = 0; d < kChanMax; ++d) {
-            const int x = lane + d * kWave;
-            v[y][d] = (ee < ne && x < vdim)
-                          ? entry_value<T>(v_cache, a.v_pool, g, e0 + ee, c * vdim + x, VW, a.VE, a.page_size) : 0.f;
+          for (int y = 0; y < 4; ++y) {
+            const int i = i0 + y * kSplitThreads;
+            if (i < units) {
+              const int e = i / upr, x = 4 * (i - e * upr);
+              *reinterpret_cast<float4*>(Vs + e * vdimp + x) = val[y];
+            }
           }
         }
+        __syncthreads();
+        if (owner) {
+          for (int e = 0; e < nsub; ++e) {
+            const float4 v4 = *reinterpret_cast<const float4*>(Vs + e * vdimp + 4 * cg);
 #pragma unroll
-        for (int y = 0; y < 4; ++y) {
-          const int ee = e + y * kWaves;
-          if (ee < ne) {
-#pragma unroll
-            for (int p = 0; p < kPairMax; ++p) {
-              if (p < pairs) {
-                const float w = wm[p * kSplitThreads + ee];
-#pragma unroll
-                for (int d = 0; d < kChanMax; ++d) acc[p][d] = fmaf(w, v[y][d], acc[p][d]);
+            for (int pp = 0; pp < kOwnMax; ++pp) {
+              const int p = pg * PP + pp;
+              if (pp < PP && p < pairs) {
+                const float w = wm[p * kSplitThreads + sub + e];
+                acc[pp][0] = fmaf(w, v4.x, acc[pp][0]);
+                acc[pp][1] = fmaf(w, v4.y, acc[pp][1]);
+                acc[pp][2] = fmaf(w, v4.z, acc[pp][2]);
+                acc[pp][3] = fmaf(w, v4.w, acc[pp][3]);
               }
             }
           }
         }
+        __syncthreads();        // before the next stage overwrites the values (and the next chunk the weights)
       }
     }
-    // add the waves' sums
-    __syncthreads();
+    if (owner) {
 #pragma unroll
-    for (int p = 0; p < kPairMax; ++p) {
-      if (p < pairs) {
+      for (int pp = 0; pp < kOwnMax; ++pp) {
+        const int p = pg * PP + pp;
+        if (pp < PP && p < pairs) {
+          const int t = p / group, h = p % group;
 #pragma unroll
-        for (int d = 0; d < kChanMax; ++d) {
-          const int x = lane + d * kWave;
-          if (x < vdim) red[(wave * pairs + p) * vdim + x] = acc[p][d];
+          for (int y = 0; y < 4; ++y) {
+            const int x = 4 * cg + y;
+            if (x < vdim) {
+              const size_t at = (size_t)(g.row + t) * H * vdim + (c * group + h) * vdim + x;
+              if (a.S == 1) Elem<T>::store(out + at, acc[pp][y]);
+              else a.part_o[(size_t)split * a.N * H * vdim + at] = acc[pp][y];
+            }
+          }
         }
       }
-    }
-    __syncthreads();
-    for (int i = tid; i < pairs * vdim; i += kSplitThreads) {
-      float sum = 0.f;
-      for (int w = 0; w < kWaves; ++w) sum += red[(size_t)w * pairs * vdim + i];
-      const int x = i % vdim, p = i / vdim, t = p / group, h = p % group;
-      const size_t at = (size_t)(g.row + t) * H * vdim + (c * group + h) * vdim + x;
-      if (a.S == 1) Elem<T>::store(out + at, sum);
-      else a.part_o[(size_t)split * a.N * H * vdim + at] = sum;
     }
     row += g.tq;
   }
@@ -711,7 +764,7 @@ int launch_split(const void* q, const void* k_cache, const void* v_cache, void* 
   const dim3 grid((a.N + a.TQ - 1) / a.TQ, a.G, a.S);
   const size_t lds_a = ((size_t)a.TQ * group * a.dim + (kSplitThreads / kWave) * kPairMax * 2) * 4;
   // (the shares' statistics are merged in the space of the mixed weights and the waves' sums)
-  const size_t work = (size_t)a.TQ * group * kSplitThreads + (size_t)(kSplitThreads / kWave) * a.TQ * group * a.vdim;
+  const size_t work = (size_t)a.TQ * group * kSplitThreads + (size_t)kStage * ((a.vdim + 3) & ~3);
   const size_t stats = (size_t)2 * a.TQ * a.H * a.S;
   const size_t lds_b = ((size_t)2 * a.TQ * a.H + (size_t)group * a.H + (work > stats ? work : stats)) * 4;
   if (lds_a > 150 * 1024 || lds_b > 150 * 1024) return -3;
@@ -840,7 +893,7 @@ TK_API int tk_pooled_window_attention_split(int dtype, const void* q, const void
                                             int dim, int vdim, int size, int pool, int page_size, int TQ, int S,
                                             int Emax, float scale, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (H < 1 || G < 1 || H % G || H / G > kGroupMax || dim < 1 || vdim < 1 || vdim > kChanMax * kWave || size < 1 ||
+  if (H < 1 || G < 1 || H % G || H / G > kGroupMax || dim < 1 || vdim < 1 || vdim > 256 || size < 1 ||
       pool < 1 || page_size < 1 || TQ < 1 || TQ > kTileMax || TQ * (H / G) > kPairMax || S < 1 || Emax < 1 ||
       (long)KE * pool < (long)G * dim || (long)VE * pool < (long)G * vdim)
     return -2;

@@ -590,7 +590,7 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
     longest_context = quarter_octave_at_least(longest_context, 64)
     rows = 1 if longest_span <= 1 else max(1, min(8, POOLED_SPLIT_PAIRS // group))
     def values_lds(rows: int) -> int:       # (the statistics of up to 4,096 (row, head, share) triples are merged in the work space)
-        return 4 * (2 * rows * num_heads + group * num_heads + max(rows * group * (256 + 4 * vdim), 2 * 4096))
+        return 4 * (2 * rows * num_heads + group * num_heads + max(rows * group * 256 + 64 * (vdim + 3), 2 * 4096))
 
     while rows > 1 and values_lds(rows) > POOLED_SPLIT_LDS:
         rows //= 2
