@@ -335,13 +335,14 @@ __global__ void pooled_window_attention_kernel(const T* __restrict__ q, const T*
 
 
 // ---------------------------------------------------------------------------
-// The same attention in three kernels that fill the GPU whatever the step's shape: a block
+// The same attention in four kernels that fill the GPU whatever the step's shape: a block
 // takes up to TQ consecutive rows of one request, ONE kv head and one share of the entries.
 //   scores:  a lane an entry: its key row (or block mean) against the queries of the kv head's
 //            query heads; raw scores to memory [row][entry][head], and every (row, head)'s
 //            maximum and sum of exponentials over the share.
-//   values:  merges the shares' statistics of ALL heads, turns the scores of its entries into
-//            normalised weights, mixes them for its own query heads, and applies them to its
+//   normalize: merges the shares' statistics and turns the scores of ALL heads into normalised
+//            weights, in place (the mixing needs every head's, so each is formed once).
+//   values:  mixes the weights of its entries for its own query heads, and applies them to its
 //            kv head's values (64 entries staged in LDS at a time; a thread owns four channels of a few
 //            (row, head) pairs); float32 partial outputs.
 //   merge:   adds the shares' partial outputs.
@@ -542,6 +543,72 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_scores_kernel(const T* _
   }
 }
 
+// scores -> normalised weights, in place, for ALL heads of a row (every kv head's value kernel
+// mixes all of them, so each is formed once here): a block a (row, 256 entries); the shares'
+// maxima and sums of the row's heads are loaded side by side and merged in LDS first.
+__global__ __launch_bounds__(kSplitThreads) void pooled_normalize_kernel(SplitArgs a) {
+  extern __shared__ float lds[];
+  const int H = a.H, S = a.S;
+  float* sm_ = lds;                 // [H][S] maxima, then as many sums
+  float* mh = sm_ + 2 * H * S;      // [H]
+  float* il = mh + H;               // [H]
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int count = H * S;
+  const size_t from = (size_t)row * count;
+  for (int i = tid; i < count; i += kSplitThreads) {
+    sm_[i] = a.part_m[from + i];
+    sm_[count + i] = a.part_l[from + i];
+  }
+  __syncthreads();
+  for (int h = tid; h < H; h += kSplitThreads) {
+    float m_all = -INFINITY;
+    for (int sh = 0; sh < S; ++sh) m_all = fmaxf(m_all, sm_[h * S + sh]);
+    float l_all = 0.f;
+    for (int sh = 0; sh < S; ++sh) {
+      const float ms = sm_[h * S + sh];
+      if (ms > -INFINITY) l_all += sm_[count + h * S + sh] * expf(ms - m_all);
+    }
+    mh[h] = m_all;
+    il[h] = 1.f / l_all;
+  }
+  __syncthreads();
+  // the entries of the row's segment (the rows of its request inside its tile), as the score kernel numbers them
+  const int r = a.req_of_token[row];
+  const int tile = row / a.TQ * a.TQ;
+  const int seg_start = max(tile, a.q_start[r]), seg_end = min(min(a.N, tile + a.TQ), a.q_start[r + 1]);
+  const int i0 = a.positions[row] - (row - seg_start), i_last = a.positions[row] + (seg_end - 1 - row);
+  const int behind = i_last - a.size - (a.pool - 1);
+  const int E = (behind >= 0 ? behind / a.pool + 1 : 0) + i_last - max(0, i0 - a.size + 1) + 1;
+  const int e = blockIdx.y * kSplitThreads + tid;
+  if (e >= E) return;
+  float* sc = a.scores + ((size_t)row * a.Emax + e) * H;
+  if (H % 4 == 0) {
+    for (int h0 = 0; h0 < H; h0 += 32) {
+      float4 v[8];
+#pragma unroll
+      for (int y = 0; y < 8; ++y)
+        if (h0 + 4 * y < H) v[y] = *reinterpret_cast<const float4*>(sc + h0 + 4 * y);
+#pragma unroll
+      for (int y = 0; y < 8; ++y) {
+        if (h0 + 4 * y < H) {
+          const int h = h0 + 4 * y;
+          float4 w;
+          w.x = v[y].x > -INFINITY ? expf(v[y].x - mh[h]) * il[h] : 0.f;
+          w.y = v[y].y > -INFINITY ? expf(v[y].y - mh[h + 1]) * il[h + 1] : 0.f;
+          w.z = v[y].z > -INFINITY ? expf(v[y].z - mh[h + 2]) * il[h + 2] : 0.f;
+          w.w = v[y].w > -INFINITY ? expf(v[y].w - mh[h + 3]) * il[h + 3] : 0.f;
+          *reinterpret_cast<float4*>(sc + h) = w;
+        }
+      }
+    }
+  } else {
+    for (int h = 0; h < H; ++h) {
+      const float v = sc[h];
+      sc[h] = v > -INFINITY ? expf(v - mh[h]) * il[h] : 0.f;
+    }
+  }
+}
+
 constexpr int kStage = 64;     // entries whose values are staged in LDS at once
 constexpr int kOwnMax = 8;     // (row, head) pairs a thread of the value kernel owns
 
@@ -579,9 +646,7 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
   extern __shared__ float lds[];
   const int H = a.H, group = a.H / a.G, vdim = a.vdim, VW = a.G * a.vdim;
   const int c = blockIdx.y, split = blockIdx.z;
-  float* mh = lds;                                   // [TQ][H]  maximum of every head
-  float* il = mh + a.TQ * H;                         // [TQ][H]  1 / sum
-  float* tk_ = il + a.TQ * H;                        // [group][H]
+  float* tk_ = lds;                                  // [group][H]
   float* wm = tk_ + group * H;                       // [TQ * group][kSplitThreads] mixed weights of a chunk
   const int vdimp = (vdim + 3) & ~3, upr = vdimp / 4;   // a row padded to pieces of four channels
   float* Vs = wm + a.TQ * group * kSplitThreads;     // [kStage][vdimp] values of a stage
@@ -600,29 +665,6 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
   while (row < row_end) {
     const Segment g = segment_at(a, row, row_end);
     const int pairs = g.tq * group;
-    __syncthreads();
-    // the shares' statistics of every (row, head): loaded side by side, merged from LDS
-    {
-      float* sm_ = wm;                                 // [tq * H][S] maxima, then as many sums
-      const int count = g.tq * H * a.S;
-      const size_t from = (size_t)g.row * H * a.S;     // (the rows of a segment follow one another)
-      for (int i = tid; i < count; i += kSplitThreads) {
-        sm_[i] = a.part_m[from + i];
-        sm_[count + i] = a.part_l[from + i];
-      }
-      __syncthreads();
-      for (int i = tid; i < g.tq * H; i += kSplitThreads) {
-        float m_all = -INFINITY;
-        for (int sh = 0; sh < a.S; ++sh) m_all = fmaxf(m_all, sm_[i * a.S + sh]);
-        float l_all = 0.f;
-        for (int sh = 0; sh < a.S; ++sh) {
-          const float ms = sm_[i * a.S + sh];
-          if (ms > -INFINITY) l_all += sm_[count + i * a.S + sh] * expf(ms - m_all);
-        }
-        mh[i] = m_all;
-        il[i] = 1.f / l_all;
-      }
-    }
     __syncthreads();
     const int e_lo = (int)((long)g.E * split / a.S), e_hi = (int)((long)g.E * (split + 1) / a.S);
     float acc[kOwnMax][4];
@@ -654,10 +696,7 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
                 s4 = *reinterpret_cast<const float4*>(sc + gh);
               }
               const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
-              float w[4];
-#pragma unroll
-              for (int y = 0; y < 4; ++y)
-                w[y] = sv[y] > -INFINITY ? expf(sv[y] - mh[t * H + gh + y]) * il[t * H + gh + y] : 0.f;
+              const float* w = sv;        // (normalised weights: the kernel before has seen to that)
 #pragma unroll
               for (int h = 0; h < kGroupMax; ++h) {
                 if (h < group) {
@@ -668,8 +707,7 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
             }
           } else {
             for (int gh = 0; gh < H; ++gh) {
-              const float s = sc[gh];
-              const float w = s > -INFINITY ? expf(s - mh[t * H + gh]) * il[t * H + gh] : 0.f;
+              const float w = sc[gh];
 #pragma unroll
               for (int h = 0; h < kGroupMax; ++h)
                 if (h < group) mixed[h] = fmaf(tk_[h * H + gh], w, mixed[h]);
@@ -763,11 +801,10 @@ int launch_split(const void* q, const void* k_cache, const void* v_cache, void* 
   const int group = a.H / a.G;
   const dim3 grid((a.N + a.TQ - 1) / a.TQ, a.G, a.S);
   const size_t lds_a = ((size_t)a.TQ * group * a.dim + (kSplitThreads / kWave) * kPairMax * 2) * 4;
-  // (the shares' statistics are merged in the space of the mixed weights and the waves' sums)
   const size_t work = (size_t)a.TQ * group * kSplitThreads + (size_t)kStage * ((a.vdim + 3) & ~3);
-  const size_t stats = (size_t)2 * a.TQ * a.H * a.S;
-  const size_t lds_b = ((size_t)2 * a.TQ * a.H + (size_t)group * a.H + (work > stats ? work : stats)) * 4;
-  if (lds_a > 150 * 1024 || lds_b > 150 * 1024) return -3;
+  const size_t lds_b = ((size_t)group * a.H + work) * 4;
+  const size_t lds_n = ((size_t)2 * a.H * a.S + 2 * a.H) * 4;
+  if (lds_a > 150 * 1024 || lds_b > 150 * 1024 || lds_n > 64 * 1024) return -3;
   static bool allowed = false;      // (per instantiation: once per storage type)
   if (!allowed) {
     hipError_t err = hipFuncSetAttribute((const void*)pooled_scores_kernel<T>,
@@ -779,6 +816,7 @@ int launch_split(const void* q, const void* k_cache, const void* v_cache, void* 
     allowed = true;
   }
   pooled_scores_kernel<T><<<grid, kSplitThreads, lds_a, stream>>>((const T*)q, (const T*)k_cache, a);
+  pooled_normalize_kernel<<<dim3(a.N, (a.Emax + kSplitThreads - 1) / kSplitThreads), kSplitThreads, lds_n, stream>>>(a);
   pooled_values_kernel<T><<<grid, kSplitThreads, lds_b, stream>>>((const T*)v_cache, (T*)out, a);
   if (a.S > 1) {
     const size_t total = (size_t)a.N * a.H * a.vdim;

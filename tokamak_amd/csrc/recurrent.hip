@@ -60,6 +60,18 @@ __global__ void tanh_kernel(const void* __restrict__ in, int f32, int parts, lon
 
 constexpr int kScanTokens = 8;   // tokens whose operands are staged in LDS at once
 
+// an operand [N, heads * dim]: T, or float32, or float32 partial sums of a split product
+struct ScanIn {
+  const void* p;
+  int f32, parts;
+  long stride;
+};
+
+template <typename T>
+__device__ __forceinline__ float scan_load(const ScanIn& in, size_t idx) {
+  return load_in<T>(in.p, in.f32, in.parts, in.stride, idx);
+}
+
 struct ScanShape {
   int heads, dim, columns, slices, slice;   // threads = columns * slices; a thread owns `slice` key channels of a column
 };
@@ -70,8 +82,7 @@ struct ScanShape {
 // outputs meet in LDS.  Tokens run in order, eight staged at a time.
 template <typename T, int SLICE>
 __global__ __launch_bounds__(1024) void wkv_scan_kernel(
-    const T* __restrict__ r_in, const T* __restrict__ k_in, const T* __restrict__ v_in,
-    const T* __restrict__ g_in, const void* __restrict__ d_in, int d_f32, int d_parts, long d_stride,
+    ScanIn r_in, ScanIn k_in, ScanIn v_in, ScanIn g_in, ScanIn d_in,
     const float* __restrict__ w0, const float* __restrict__ u, const float* __restrict__ gain,
     float* __restrict__ state, const int* __restrict__ q_start, const int* __restrict__ state_slots,
     T* __restrict__ out, ScanShape sh, float eps) {
@@ -107,16 +118,16 @@ __global__ __launch_bounds__(1024) void wkv_scan_kernel(
     for (int i = tid; i < tb * dim; i += nthreads) {
       const int t = i / dim, c = i - t * dim;
       const size_t at = (size_t)(t0 + t) * HD + base + c;
-      const float kv = Elem<T>::load(k_in + at);
-      rr[t * dimp + c] = Elem<T>::load(r_in + at);
+      const float kv = scan_load<T>(k_in, at);
+      rr[t * dimp + c] = scan_load<T>(r_in, at);
       kk[t * dimp + c] = kv;
       uk[t * dimp + c] = u[base + c] * kv;
-      ww[t * dimp + c] = expf(-expf(load_in<T>(d_in, d_f32, d_parts, d_stride, at) + w0[base + c]));
+      ww[t * dimp + c] = expf(-expf(scan_load<T>(d_in, at) + w0[base + c]));
     }
     float vloc[TB];
 #pragma unroll
     for (int t = 0; t < TB; ++t)
-      vloc[t] = (t < tb && live) ? Elem<T>::load(v_in + (size_t)(t0 + t) * HD + base + j) : 0.f;
+      vloc[t] = (t < tb && live) ? scan_load<T>(v_in, (size_t)(t0 + t) * HD + base + j) : 0.f;
     __syncthreads();
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
@@ -162,7 +173,7 @@ __global__ __launch_bounds__(1024) void wkv_scan_kernel(
     for (int t = ks; t < tb; t += KS) {
       if (live) {
         const size_t at = (size_t)(t0 + t) * HD + base + j;
-        const float g = Elem<T>::load(g_in + at);
+        const float g = scan_load<T>(g_in, at);
         Elem<T>::store(out + at, os[t * dimp + j] * rstd[t] * gj * (g / (1.f + expf(-g))));
       }
     }
@@ -177,8 +188,7 @@ __global__ __launch_bounds__(1024) void wkv_scan_kernel(
 }
 
 template <typename T>
-int launch_scan(const void* r, const void* k, const void* v, const void* g, const void* d, int d_f32, int d_parts,
-                long d_stride, const float* w0, const float* u, const float* gain, float* state,
+int launch_scan(ScanIn r, ScanIn k, ScanIn v, ScanIn g, ScanIn d, const float* w0, const float* u, const float* gain, float* state,
                 const int* q_start, const int* state_slots, void* out, int R, int heads, int dim, float eps,
                 hipStream_t stream) {
   ScanShape sh;
@@ -202,7 +212,7 @@ int launch_scan(const void* r, const void* k, const void* v, const void* g, cons
       allowed = true;                                                                                         \
     }                                                                                                         \
     wkv_scan_kernel<T, SLICE><<<grid, threads, lds, stream>>>(                                                \
-        (const T*)r, (const T*)k, (const T*)v, (const T*)g, d, d_f32, d_parts, d_stride, w0, u, gain, state,  \
+        r, k, v, g, d, w0, u, gain, state,                                                                  \
         q_start, state_slots, (T*)out, sh, eps);                                                              \
   }
   if (sh.slice <= 4) TK_SCAN(4)
@@ -242,19 +252,24 @@ TK_API int tk_tanh(int dtype, const void* in, int in_f32, int parts, long part_s
   return launch_status();
 }
 
-// r, k, v, g, out: [N, heads * dim] in dtype; d: the decay's pre-activation, dtype or float32
-// (partial sums allowed); state [slots, heads, dim, dim] float32.  dim <= 256.
-TK_API int tk_wkv_scan(int dtype, const void* r, const void* k, const void* v, const void* g, const void* d,
-                       int d_f32, int d_parts, long d_stride, const float* w0, const float* u, const float* gain,
-                       float* state, const int* q_start, const int* state_slots, void* out, int R, int heads,
-                       int dim, float eps, hipStream_t stream) {
+// r, k, v, g (gate), d (the decay's pre-activation): [N, heads * dim] in dtype, or float32, or
+// float32 partial sums [parts, N, heads * dim]; out in dtype; state [slots, heads, dim, dim]
+// float32.  dim <= 256.
+TK_API int tk_wkv_scan(int dtype, const void* r, int r_f32, int r_parts, long r_stride, const void* k, int k_f32,
+                       int k_parts, long k_stride, const void* v, int v_f32, int v_parts, long v_stride,
+                       const void* g, int g_f32, int g_parts, long g_stride, const void* d, int d_f32, int d_parts,
+                       long d_stride, const float* w0, const float* u, const float* gain, float* state,
+                       const int* q_start, const int* state_slots, void* out, int R, int heads, int dim, float eps,
+                       hipStream_t stream) {
   if (R <= 0 || heads <= 0) return 0;
   if (dim < 1 || dim > 256) return -2;
+  const ScanIn ri{r, r_f32, r_parts, r_stride}, ki{k, k_f32, k_parts, k_stride}, vi{v, v_f32, v_parts, v_stride},
+      gi{g, g_f32, g_parts, g_stride}, di{d, d_f32, d_parts, d_stride};
   if (dtype == 0)
-    return launch_scan<float>(r, k, v, g, d, d_f32, d_parts, d_stride, w0, u, gain, state, q_start, state_slots,
-                              out, R, heads, dim, eps, stream);
-  return launch_scan<bf16_t>(r, k, v, g, d, d_f32, d_parts, d_stride, w0, u, gain, state, q_start, state_slots,
-                             out, R, heads, dim, eps, stream);
+    return launch_scan<float>(ri, ki, vi, gi, di, w0, u, gain, state, q_start, state_slots, out, R, heads, dim, eps,
+                              stream);
+  return launch_scan<bf16_t>(ri, ki, vi, gi, di, w0, u, gain, state, q_start, state_slots, out, R, heads, dim, eps,
+                             stream);
 }
 
 TK_SLOTS(tk_token_shift)

@@ -199,7 +199,8 @@ _SIGS = {
         "tk_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                            c_int, c_int, c_void_p],
         "tk_tanh": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_long, c_void_p],
-        "tk_wkv_scan": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p,
+        "tk_wkv_scan": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int,
+                        c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p,
                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
                         c_void_p],
     },
@@ -589,18 +590,18 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
     # the length rounded as recorded steps round it: a step computes the same bits recorded or not
     longest_context = quarter_octave_at_least(longest_context, 64)
     rows = 1 if longest_span <= 1 else max(1, min(8, POOLED_SPLIT_PAIRS // group))
-    def values_lds(rows: int) -> int:       # (the statistics of up to 4,096 (row, head, share) triples are merged in the work space)
-        return 4 * (2 * rows * num_heads + group * num_heads + max(rows * group * 256 + 64 * (vdim + 3), 2 * 4096))
+    def values_lds(rows: int) -> int:
+        return 4 * (group * num_heads + rows * group * 256 + 64 * (vdim + 3))
 
     while rows > 1 and values_lds(rows) > POOLED_SPLIT_LDS:
         rows //= 2
     if (values_lds(rows) > POOLED_SPLIT_LDS or 4 * (rows * group * dim + 8 * POOLED_SPLIT_PAIRS) > POOLED_SPLIT_LDS
-            or rows * num_heads > 4096):
+            or num_heads > 4096):
         return None
     most = min(longest_context, window + rows - 1) + longest_context // pool + 1
     blocks = -(-n // rows) * num_kv_heads
-    # (a share of at least 32 entries; the shares' statistics of a tile's rows and heads fit the LDS they are merged in)
-    shares = max(1, min(32, POOLED_SPLIT_BLOCKS // blocks, -(-most // 32), 4096 // (rows * num_heads)))
+    # (a share of at least 32 entries; the shares' statistics of a row's heads fit the LDS they are merged in)
+    shares = max(1, min(32, POOLED_SPLIT_BLOCKS // blocks, -(-most // 32), 4096 // num_heads))
     return rows, shares, most
 
 
@@ -688,21 +689,21 @@ def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tens
              *, heads: int, dim: int, eps: float) -> None:
     """Per request and head, over the step's tokens in order: o = (S + diag(u) k v^T)^T r, then
     S <- diag(exp(-exp(decay_in + w0))) S + k v^T (S float32 [slots, heads, dim, dim], kept);
-    out = o / rms(o) * gain * silu(gate).  r, k, v, gate, out: [N, heads * dim]."""
+    out = o / rms(o) * gain * silu(gate).  r, k, v, gate, decay_in: [N, heads * dim] in out's dtype or
+    float32, or float32 partial sums [P, N, heads * dim] of a split product."""
     _gpu(r, k, v, gate, decay_in, w0, u, gain, state, out)
     n, hd = out.shape
     dtype = out.dtype
     _need(hd == heads * dim and 1 <= dim <= WKV_MAX_DIM, f"the scan takes heads of up to {WKV_MAX_DIM} channels")
-    for t in (r, k, v, gate):
-        _need(t.shape == (n, hd) and t.dtype == dtype, "scan operands are [N, heads * dim] in one dtype")
     for t in (w0, u, gain):
         _need(t.dtype == torch.float32 and t.numel() == hd, "decay offset, bonus and gain are float32 [heads * dim]")
     _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, dim), "the state is float32 [slots, heads, dim, dim]")
     _need(batch.num_tokens == n, "the step's descriptor does not match")
-    p, is_f32, parts, stride = _branch(decay_in, n, hd, dtype, "decay_in")
-    _note(f"{n}x{heads}x{dim}", n * hd * 6 * r.element_size(), 4.0 * n * heads * dim * dim)
+    operands = [x for t, what in ((r, "r"), (k, "k"), (v, "v"), (gate, "gate"), (decay_in, "decay_in"))
+                for x in _branch(t, n, hd, dtype, what)]
+    _note(f"{n}x{heads}x{dim}", n * hd * 6 * out.element_size(), 4.0 * n * heads * dim * dim)
     _check(_fn("recurrent", "tk_wkv_scan")(
-        _code(dtype), _p(r), _p(k), _p(v), _p(gate), p, is_f32, parts, stride, _p(w0), _p(u), _p(gain), _p(state),
+        _code(dtype), *operands, _p(w0), _p(u), _p(gain), _p(state),
         _p(batch.q_start), _p(batch.state_slots), _p(out), batch.num_requests, heads, dim, float(eps), _stream()),
         "wkv_scan")
 

@@ -77,10 +77,11 @@ class DecayedStateTimeMix(Mixer):
         n = h.shape[0]
         mixes = torch.empty((len(MIXES), n, self.hidden_size), dtype=self.dtype, device=h.device)
         ops.token_shift(h, self.mu, store.state["last"], mixes, batch)
-        r, k, v, gate = (linear(mixes[i], getattr(self, s)) for i, s in enumerate(MIXES[:4]))
+        # (split products leave float32 partial sums, which the scan adds as it loads)
+        r, k, v, gate = (linear(mixes[i], getattr(self, s), allow_partials=True) for i, s in enumerate(MIXES[:4]))
         low = torch.empty((n, self.w1.shape[0]), dtype=self.dtype, device=h.device)
         ops.tanh(linear(mixes[4], self.w1, allow_partials=True), low)
-        decay_in = linear(low, self.w2, out_dtype=torch.float32)
+        decay_in = linear(low, self.w2, out_dtype=torch.float32, allow_partials=True)
         out = torch.empty((n, self.width), dtype=self.dtype, device=h.device)
         ops.wkv_scan(r, k, v, gate, decay_in, self.w0, self.u, self.gain, store.state["S"], out, batch,
                      heads=self.num_heads, dim=self.head_dim, eps=self.norm_eps)
