@@ -21,9 +21,15 @@ namespace {
 template <typename T>
 __device__ __forceinline__ float load_in(const void* p, int f32, int parts, long part_stride, size_t idx) {
   if (!f32) return Elem<T>::load(reinterpret_cast<const T*>(p) + idx);
-  const float* f = reinterpret_cast<const float*>(p);
-  float s = f[idx];
-  for (int i = 1; i < parts; ++i) s += f[idx + (size_t)i * part_stride];
+  const float* f = reinterpret_cast<const float*>(p) + idx;
+  float s = f[0];
+  int i = 1;
+  for (; i + 3 < parts; i += 4) {      // four loads in flight; the sums in the order of the parts
+    const float a = f[(size_t)i * part_stride], b = f[(size_t)(i + 1) * part_stride];
+    const float c = f[(size_t)(i + 2) * part_stride], d = f[(size_t)(i + 3) * part_stride];
+    s = (((s + a) + b) + c) + d;
+  }
+  for (; i < parts; ++i) s += f[(size_t)i * part_stride];
   return s;
 }
 
@@ -67,8 +73,10 @@ struct ScanIn {
   long stride;
 };
 
-template <typename T>
+// PLAIN: the operand is known to be T (a long portion's products): one load, no branch
+template <typename T, bool PLAIN>
 __device__ __forceinline__ float scan_load(const ScanIn& in, size_t idx) {
+  if (PLAIN) return Elem<T>::load(reinterpret_cast<const T*>(in.p) + idx);
   return load_in<T>(in.p, in.f32, in.parts, in.stride, idx);
 }
 
@@ -80,7 +88,7 @@ struct ScanShape {
 // of column j in registers: the key channels of a head are cut over `slices` groups of threads, so
 // that a token costs each thread `slice` multiply-adds and not `dim`; the groups' partial
 // outputs meet in LDS.  Tokens run in order, eight staged at a time.
-template <typename T, int SLICE>
+template <typename T, int SLICE, bool PLAIN>
 __global__ __launch_bounds__(1024) void wkv_scan_kernel(
     ScanIn r_in, ScanIn k_in, ScanIn v_in, ScanIn g_in, ScanIn d_in,
     const float* __restrict__ w0, const float* __restrict__ u, const float* __restrict__ gain,
@@ -118,16 +126,16 @@ __global__ __launch_bounds__(1024) void wkv_scan_kernel(
     for (int i = tid; i < tb * dim; i += nthreads) {
       const int t = i / dim, c = i - t * dim;
       const size_t at = (size_t)(t0 + t) * HD + base + c;
-      const float kv = scan_load<T>(k_in, at);
-      rr[t * dimp + c] = scan_load<T>(r_in, at);
+      const float kv = scan_load<T, PLAIN>(k_in, at);
+      rr[t * dimp + c] = scan_load<T, PLAIN>(r_in, at);
       kk[t * dimp + c] = kv;
       uk[t * dimp + c] = u[base + c] * kv;
-      ww[t * dimp + c] = expf(-expf(scan_load<T>(d_in, at) + w0[base + c]));
+      ww[t * dimp + c] = expf(-expf(scan_load<T, false>(d_in, at) + w0[base + c]));
     }
     float vloc[TB];
 #pragma unroll
     for (int t = 0; t < TB; ++t)
-      vloc[t] = (t < tb && live) ? scan_load<T>(v_in, (size_t)(t0 + t) * HD + base + j) : 0.f;
+      vloc[t] = (t < tb && live) ? scan_load<T, PLAIN>(v_in, (size_t)(t0 + t) * HD + base + j) : 0.f;
     __syncthreads();
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
@@ -173,7 +181,7 @@ __global__ __launch_bounds__(1024) void wkv_scan_kernel(
     for (int t = ks; t < tb; t += KS) {
       if (live) {
         const size_t at = (size_t)(t0 + t) * HD + base + j;
-        const float g = scan_load<T>(g_in, at);
+        const float g = scan_load<T, PLAIN>(g_in, at);
         Elem<T>::store(out + at, os[t * dimp + j] * rstd[t] * gj * (g / (1.f + expf(-g))));
       }
     }
@@ -202,22 +210,28 @@ int launch_scan(ScanIn r, ScanIn k, ScanIn v, ScanIn g, ScanIn d, const float* w
   const int dimp = (dim + 3) & ~3;
   const size_t lds = ((size_t)5 * kScanTokens * dimp + kScanTokens + (size_t)sh.slices * kScanTokens * sh.columns) * 4;
   const dim3 grid(R, heads);
-#define TK_SCAN(SLICE)                                                                                        \
+  const bool plain = !r.f32 && !k.f32 && !v.f32 && !g.f32;
+#define TK_SCAN_AS(SLICE, PLAIN)                                                                              \
   {                                                                                                           \
     static bool allowed = false;                                                                              \
     if (!allowed) {                                                                                           \
-      const hipError_t err = hipFuncSetAttribute((const void*)wkv_scan_kernel<T, SLICE>,                      \
+      const hipError_t err = hipFuncSetAttribute((const void*)wkv_scan_kernel<T, SLICE, PLAIN>,               \
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);     \
       if (err != hipSuccess) return (int)err;                                                                 \
       allowed = true;                                                                                         \
     }                                                                                                         \
-    wkv_scan_kernel<T, SLICE><<<grid, threads, lds, stream>>>(                                                \
-        r, k, v, g, d, w0, u, gain, state,                                                                  \
-        q_start, state_slots, (T*)out, sh, eps);                                                              \
+    wkv_scan_kernel<T, SLICE, PLAIN><<<grid, threads, lds, stream>>>(r, k, v, g, d, w0, u, gain, state,       \
+                                                                     q_start, state_slots, (T*)out, sh, eps); \
+  }
+#define TK_SCAN(SLICE)                 \
+  {                                    \
+    if (plain) TK_SCAN_AS(SLICE, true) \
+    else TK_SCAN_AS(SLICE, false)      \
   }
   if (sh.slice <= 4) TK_SCAN(4)
   else if (sh.slice <= 16) TK_SCAN(16)
   else TK_SCAN(64)
+#undef TK_SCAN_AS
 #undef TK_SCAN
   return launch_status();
 }
