@@ -263,6 +263,38 @@ def test_mixed_batches_with_pages_and_slots_used_again(models, name, dtype):
     assert worst <= LIMIT[dtype], (name, dtype, worst, where)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_kernel_form_of_the_attention(models, dtype, monkeypatch):
+    """The form for sizes the four-kernel form does not take (more than 16 query heads a kv
+    head, more than 256 value channels), forced here on a small shape: every cutting, and a
+    wide group for real."""
+    from tokamak_amd.kernels import ops
+
+    monkeypatch.setattr(ops, "POOLED_ONE_KERNEL_ONLY", True)
+    runner, cfg, w = runner_for(models, "odd", dtype, use_graphs=False)
+    requests = requests_for(cfg, seed=3)
+    expected = expected_for(cfg, w, requests, dtype)
+    for steps in (whole(requests), tail_one_by_one("r4", requests["r4"]), portions("r4", requests["r4"])):
+        worst, where = worst_error(steps, run_steps(runner, steps), expected)
+        assert worst <= LIMIT[dtype], (dtype, worst, where)
+    monkeypatch.setattr(ops, "POOLED_ONE_KERNEL_ONLY", False)
+    assert ops.pooled_split_plan(34, 2, 8, 8, 6, 3, 10, 10, 100) is None       # 17 heads a kv head
+
+
+def test_a_group_of_seventeen_heads(tmp_path):
+    from tokamak_amd.engine.runner import ModelRunner
+
+    cfg = model_json([layer(heads=17, kv_heads=1, dim=8, vdim=8, window=6, pool=3)], vocab=50, width=40)
+    w = random_weights(cfg, seed=9)
+    folder = write_folder(tmp_path / "g17", cfg, w)
+    toks = tokens(50, 70, 4)
+    runner = ModelRunner.from_folder(folder, dtype="float32", page_size=16, kv_pool_tokens=128, max_requests=2)
+    expected = {"x": oracle_logits(cfg, w, toks)}
+    for steps in (whole({"x": toks}), tail_one_by_one("x", toks, tail=20)):
+        worst, where = worst_error(steps, run_steps(runner, steps), expected)
+        assert worst <= LIMIT["float32"], (worst, where)
+
+
 def test_window_and_pool_edges_show(tmp_path):
     """Attention so sharp (scores times eight) that a key which is one position inside or
     outside the window, or a block that is pooled one step early or late, moves the logits by

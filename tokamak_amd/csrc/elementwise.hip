@@ -604,11 +604,55 @@ __global__ void scaled_sum_kernel(const void* __restrict__ a, int a_f32, int a_p
   out[idx] = v;
 }
 
+// four consecutive columns a thread: H a multiple of 4 (every row then starts on a border of four)
+template <typename T>
+__device__ __forceinline__ float4 branch_four(const void* p, int f32, int parts, long part_stride, size_t idx) {
+  if (!f32) return Load4<T>::at(reinterpret_cast<const T*>(p) + idx);
+  const float* f = reinterpret_cast<const float*>(p) + idx;
+  float4 s = *reinterpret_cast<const float4*>(f);
+  for (int i = 1; i < parts; ++i) {
+    const float4 a = *reinterpret_cast<const float4*>(f + (size_t)i * part_stride);
+    s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+  }
+  return s;
+}
+
+template <typename T>
+__global__ void scaled_sum_four_kernel(const void* __restrict__ a, int a_f32, int a_parts, long a_stride, float wa,
+                                       const void* __restrict__ b, int b_f32, int b_parts, long b_stride, float wb,
+                                       const float* __restrict__ scale, float* __restrict__ out, int H, size_t total4) {
+  const size_t i4 = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i4 >= total4) return;
+  const size_t idx = i4 * 4;
+  const float4 x = branch_four<T>(a, a_f32, a_parts, a_stride, idx);
+  float4 v = make_float4(wa * x.x, wa * x.y, wa * x.z, wa * x.w);
+  if (b != nullptr) {
+    const float4 y = branch_four<T>(b, b_f32, b_parts, b_stride, idx);
+    v = make_float4(fmaf(wb, y.x, v.x), fmaf(wb, y.y, v.y), fmaf(wb, y.z, v.z), fmaf(wb, y.w, v.w));
+  }
+  if (scale != nullptr) {
+    const float4 g = *reinterpret_cast<const float4*>(scale + idx % H);
+    v = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+  }
+  *reinterpret_cast<float4*>(out + idx) = v;
+}
+
 TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long a_stride, float wa,
                          const void* b, int b_f32, int b_parts, long b_stride, float wb, const float* scale,
                          float* out, int N, int H, hipStream_t stream) {
   if (N <= 0 || H <= 0) return 0;
   const size_t total = (size_t)N * H;
+  if (H % 4 == 0 && a_stride % 4 == 0 && b_stride % 4 == 0) {
+    const size_t total4 = total / 4;
+    const unsigned blocks4 = (unsigned)((total4 + 255) / 256);
+    if (dtype == 0)
+      scaled_sum_four_kernel<float><<<blocks4, 256, 0, stream>>>(a, a_f32, a_parts, a_stride, wa, b, b_f32, b_parts,
+                                                                 b_stride, wb, scale, out, H, total4);
+    else
+      scaled_sum_four_kernel<bf16_t><<<blocks4, 256, 0, stream>>>(a, a_f32, a_parts, a_stride, wa, b, b_f32, b_parts,
+                                                                  b_stride, wb, scale, out, H, total4);
+    return launch_status();
+  }
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == 0)
     scaled_sum_kernel<float><<<blocks, 256, 0, stream>>>(a, a_f32, a_parts, a_stride, wa, b, b_f32, b_parts,

@@ -33,6 +33,30 @@ __device__ __forceinline__ float load_in(const void* p, int f32, int parts, long
   return s;
 }
 
+// VEC consecutive elements of T as one 16-byte access (VEC = 4 float32 or 8 bfloat16)
+template <typename T, int VEC> __device__ __forceinline__ void load_vec(const T* p, float* o);
+template <> __device__ __forceinline__ void load_vec<float, 4>(const float* p, float* o) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+template <> __device__ __forceinline__ void load_vec<bf16_t, 8>(const bf16_t* p, float* o) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+template <typename T, int VEC> __device__ __forceinline__ void store_vec(T* p, const float* o);
+template <> __device__ __forceinline__ void store_vec<float, 4>(float* p, const float* o) {
+  *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+template <> __device__ __forceinline__ void store_vec<bf16_t, 8>(bf16_t* p, const float* o) {
+  *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]),
+                                            pack_bf16x2(o[6], o[7]));
+}
+
 template <typename T>
 __global__ void token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu,
                                    float* __restrict__ last, T* __restrict__ out,
@@ -54,6 +78,51 @@ __global__ void token_shift_kernel(const T* __restrict__ h, const float* __restr
     Elem<T>::store(out + ((size_t)s * N + n) * W + c, cur + d * mu[(size_t)s * W + c]);
   // the thread that has read the old row of the state is the one that replaces it
   if (head) mine[c] = newest;
+}
+
+// The same, a thread VEC consecutive columns (16 bytes of a row of T): W a multiple of VEC.
+template <typename T, int VEC>
+__global__ void token_shift_vec_kernel(const T* __restrict__ h, const float* __restrict__ mu,
+                                       float* __restrict__ last, T* __restrict__ out,
+                                       const int* __restrict__ req_of_token, const int* __restrict__ q_start,
+                                       const int* __restrict__ state_slots, int N, int W, int S) {
+  const int n = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+  if (c >= W) return;
+  const int r = req_of_token[n];
+  const int first = q_start[r];
+  const int end = q_start[r + 1];
+  const bool head = n == first;
+  float* mine = last + (size_t)state_slots[r] * W;
+  float cur[VEC], prev[VEC], newest[VEC];
+  load_vec<T, VEC>(h + (size_t)n * W + c, cur);
+  if (head) {
+#pragma unroll
+    for (int y = 0; y < VEC; y += 4) {
+      const float4 v = *reinterpret_cast<const float4*>(mine + c + y);
+      prev[y] = v.x; prev[y + 1] = v.y; prev[y + 2] = v.z; prev[y + 3] = v.w;
+    }
+    load_vec<T, VEC>(h + (size_t)(end - 1) * W + c, newest);
+  } else {
+    load_vec<T, VEC>(h + (size_t)(n - 1) * W + c, prev);
+  }
+  for (int s = 0; s < S; ++s) {
+    float o[VEC];
+#pragma unroll
+    for (int y = 0; y < VEC; y += 4) {
+      const float4 m = *reinterpret_cast<const float4*>(mu + (size_t)s * W + c + y);
+      o[y] = cur[y] + (prev[y] - cur[y]) * m.x;
+      o[y + 1] = cur[y + 1] + (prev[y + 1] - cur[y + 1]) * m.y;
+      o[y + 2] = cur[y + 2] + (prev[y + 2] - cur[y + 2]) * m.z;
+      o[y + 3] = cur[y + 3] + (prev[y + 3] - cur[y + 3]) * m.w;
+    }
+    store_vec<T, VEC>(out + ((size_t)s * N + n) * W + c, o);
+  }
+  if (head) {
+#pragma unroll
+    for (int y = 0; y < VEC; y += 4)
+      *reinterpret_cast<float4*>(mine + c + y) = make_float4(newest[y], newest[y + 1], newest[y + 2], newest[y + 3]);
+  }
 }
 
 template <typename T>
@@ -244,6 +313,19 @@ TK_API int tk_token_shift(int dtype, const void* h, const float* mu, float* last
                           const int* req_of_token, const int* q_start, const int* state_slots, int N, int W,
                           int S, hipStream_t stream) {
   if (N <= 0 || W <= 0 || S <= 0) return 0;
+  const int vec = dtype == 0 ? 4 : 8;
+  if (W % vec == 0) {      // (rows, the state's rows and the mix weights then all start on 16-byte borders)
+    const int columns = W / vec;
+    const int threads = columns >= 256 ? 256 : 64;
+    const dim3 grid(N, (columns + threads - 1) / threads);
+    if (dtype == 0)
+      token_shift_vec_kernel<float, 4><<<grid, threads, 0, stream>>>((const float*)h, mu, last, (float*)out,
+                                                                     req_of_token, q_start, state_slots, N, W, S);
+    else
+      token_shift_vec_kernel<bf16_t, 8><<<grid, threads, 0, stream>>>((const bf16_t*)h, mu, last, (bf16_t*)out,
+                                                                      req_of_token, q_start, state_slots, N, W, S);
+    return launch_status();
+  }
   const int threads = W >= 256 ? 256 : 64;
   const dim3 grid(N, (W + threads - 1) / threads);
   if (dtype == 0)

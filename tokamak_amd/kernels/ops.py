@@ -569,6 +569,8 @@ def pooled_window_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, l
     return rows, chunk, threads
 
 
+POOLED_ONE_KERNEL_ONLY = False   # tests set this to run the one-kernel form on sizes the other form takes
+
 POOLED_SPLIT_GROUP = 16      # query heads a kv head, value channels and rows times heads a block
 POOLED_SPLIT_VDIM = 256      # that the three-kernel form of the attention takes
 POOLED_SPLIT_PAIRS = 32
@@ -585,7 +587,7 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
     from tokamak_amd.kernels.attention import quarter_octave_at_least
 
     group = num_heads // num_kv_heads
-    if group > POOLED_SPLIT_GROUP or vdim > POOLED_SPLIT_VDIM:
+    if group > POOLED_SPLIT_GROUP or vdim > POOLED_SPLIT_VDIM or POOLED_ONE_KERNEL_ONLY:
         return None
     # the length rounded as recorded steps round it: a step computes the same bits recorded or not
     longest_context = quarter_octave_at_least(longest_context, 64)
