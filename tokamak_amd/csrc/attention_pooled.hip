@@ -140,12 +140,28 @@ __global__ __launch_bounds__(1024) void bias_norm_store_row_kernel(
       if (c < total) x[u] += Elem<T>::load(reinterpret_cast<const T*>(qkv) + row + c);
     }
   } else {
-    const float* f = reinterpret_cast<const float*>(qkv);
-    for (int i = 0; i < parts; ++i) {
+    // partial sums of a split product: four parts' loads asked for together, added in the parts' order
+    const float* f = reinterpret_cast<const float*>(qkv) + row;
+    int i = 0;
+    for (; i + 3 < parts; i += 4) {
+      float y[4][kRowRegs];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int u = 0; u < kRowRegs; ++u) {
+          const int c = threadIdx.x + u * blockDim.x;
+          y[j][u] = c < total ? f[c + (size_t)(i + j) * part_stride] : 0.f;
+        }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int u = 0; u < kRowRegs; ++u) x[u] += y[j][u];
+    }
+    for (; i < parts; ++i) {
 #pragma unroll
       for (int u = 0; u < kRowRegs; ++u) {
         const int c = threadIdx.x + u * blockDim.x;
-        if (c < total) x[u] += f[row + c + (size_t)i * part_stride];
+        if (c < total) x[u] += f[c + (size_t)i * part_stride];
       }
     }
   }
