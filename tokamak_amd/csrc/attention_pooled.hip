@@ -559,6 +559,164 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_scores_kernel(const T* _
   }
 }
 
+// The score kernel on the matrix cores (bfloat16 storage, dim a multiple of 16, rows on 16-byte
+// borders).  A wave takes 32 token entries at a time: S^T[entry][pair] = K[entry][:] . Q[pair][:]
+// with v_mfma_f32_32x32x16_bf16, A = 32 key rows x 16 channels straight from the pages (lane
+// (col, g) loads channels [16 c + 8 g, + 8) of entry col's row), B = the tile's queries, kept in
+// registers for the whole walk (pair col = row * group + head; pairs beyond the tile's are
+// zero).  A lane then holds, for its pair, the entries 8 i + 4 g + j (i, j < 4) of the 32.  The
+// products of bfloat16 numbers are exact in float32 and are added in float32.  The few block
+// means (float32) keep the vector path above, by the same lanes, before the tokens.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+union KeyFrag {
+  uint4 u;
+  bf16x8_t v;
+};
+constexpr int kStepsMax = 16;   // 16-channel steps: dim <= 256
+
+__global__ __launch_bounds__(kSplitThreads) void pooled_scores_mfma_kernel(const bf16_t* __restrict__ q,
+                                                                           const bf16_t* __restrict__ k_cache,
+                                                                           SplitArgs a) {
+  extern __shared__ float lds[];
+  const int group = a.H / a.G, dim = a.dim, KW = a.G * a.dim, steps = dim / 16;
+  const int c = blockIdx.y, split = blockIdx.z;
+  float* qs = lds;                                   // [TQ][group][dim] (for the block means)
+  float* red = qs + a.TQ * group * dim;              // [2 waves' worth][kPairMax][2]
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  constexpr int kWaves = kSplitThreads / kWave;
+  const int col = lane & 31, g = lane >> 5;
+  const int row_end = min(a.N, (int)(blockIdx.x + 1) * a.TQ);
+  int row = blockIdx.x * a.TQ;
+  while (row < row_end) {
+    const Segment sg = segment_at(a, row, row_end);
+    const int pairs = sg.tq * group;
+    __syncthreads();
+    for (int i = tid; i < pairs * dim; i += kSplitThreads) {
+      const int x = i % dim, tg = i / dim, t = tg / group, h = tg % group;
+      qs[i] = Elem<bf16_t>::load(q + (size_t)(sg.row + t) * a.H * dim + (c * group + h) * dim + x);
+    }
+    // this lane's pair and its query fragments
+    const bool pair_live = col < pairs;
+    const int my_t = col / group, my_h = col % group;
+    const int my_i = sg.i0 + my_t;
+    KeyFrag qreg[kStepsMax];
+#pragma unroll
+    for (int s = 0; s < kStepsMax; ++s) {
+      qreg[s].u = make_uint4(0, 0, 0, 0);
+      if (s < steps && pair_live)
+        qreg[s].u = *reinterpret_cast<const uint4*>(q + (size_t)(sg.row + my_t) * a.H * dim + (c * group + my_h) * dim +
+                                                    16 * s + 8 * g);
+    }
+    __syncthreads();
+    const int e_lo = (int)((long)sg.E * split / a.S), e_hi = (int)((long)sg.E * (split + 1) / a.S);
+    // --- block means: a lane an entry, every pair (few entries; float32 throughout) ---
+    float m[kPairMax], l[kPairMax];
+#pragma unroll
+    for (int p = 0; p < kPairMax; ++p) {
+      m[p] = -INFINITY;
+      l[p] = 0.f;
+    }
+    const int pooled_hi = min(e_hi, sg.NB);
+    for (int entry = e_lo + tid; entry < pooled_hi; entry += kSplitThreads) {
+      float acc[kPairMax];
+#pragma unroll
+      for (int p = 0; p < kPairMax; ++p) acc[p] = 0.f;
+      for (int x = 0; x < dim; ++x) {
+        const float kx = a.k_pool[pooled_at(sg.table, entry, c * dim + x, KW, a.KE, a.page_size)];
+#pragma unroll
+        for (int p = 0; p < kPairMax; ++p)
+          if (p < pairs) acc[p] = fmaf(qs[p * dim + x], kx, acc[p]);
+      }
+#pragma unroll
+      for (int p = 0; p < kPairMax; ++p) {
+        if (p < pairs) {
+          const int t = p / group, h = p % group;
+          const bool seen = entry_seen(a, sg, entry, sg.i0 + t);
+          const float sc = seen ? acc[p] * a.scale : -INFINITY;
+          a.scores[((size_t)(sg.row + t) * a.Emax + entry) * a.H + c * group + h] = sc;
+          if (seen) {
+            const float m_new = fmaxf(m[p], sc);
+            l[p] = l[p] * expf(m[p] - m_new) + expf(sc - m_new);
+            m[p] = m_new;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < kPairMax; ++p) {
+      if (p < pairs) {
+        const float m_all = wave_max(m[p]);
+        const float l_all = wave_sum(m[p] > -INFINITY ? l[p] * expf(m[p] - m_all) : 0.f);
+        if (lane == 0) {
+          red[(wave * kPairMax + p) * 2] = m_all;
+          red[(wave * kPairMax + p) * 2 + 1] = l_all;
+        }
+      }
+    }
+    // --- tokens: 32 entries a wave and turn, on the matrix cores ---
+    const int t_lo = max(e_lo, sg.NB);
+    float mm = -INFINITY, ll = 0.f;      // of this lane's pair over the entries it holds
+    for (int e0 = t_lo + 32 * wave; e0 < e_hi; e0 += 32 * kWaves) {
+      const int mine = min(e0 + col, e_hi - 1);       // (a row that exists; what lies past the share is not used)
+      const int pos = sg.j0 + mine - sg.NB;
+      const bf16_t* rowp = k_cache + ((size_t)sg.table[pos / a.page_size] * a.page_size + pos % a.page_size) * KW +
+                           (size_t)c * dim + 8 * g;
+      KeyFrag kf[kStepsMax];
+#pragma unroll
+      for (int s = 0; s < kStepsMax; ++s)
+        if (s < steps) kf[s].u = *reinterpret_cast<const uint4*>(rowp + 16 * s);
+      float16_t acc;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) acc[x] = 0.f;
+#pragma unroll
+      for (int s = 0; s < kStepsMax; ++s)
+        if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s].v, qreg[s].v, acc, 0, 0, 0);
+      if (pair_live) {
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+          const int entry = e0 + 8 * (x >> 2) + 4 * g + (x & 3);
+          if (entry < e_hi) {
+            const int j = sg.j0 + entry - sg.NB;
+            const bool seen = j <= my_i && my_i - j < a.size;
+            const float sc = seen ? acc[x] * a.scale : -INFINITY;
+            a.scores[((size_t)(sg.row + my_t) * a.Emax + entry) * a.H + c * group + my_h] = sc;
+            if (seen) {
+              const float m_new = fmaxf(mm, sc);
+              ll = ll * expf(mm - m_new) + expf(sc - m_new);
+              mm = m_new;
+            }
+          }
+        }
+      }
+    }
+    {   // the two halves of the wave hold the same pairs
+      const float m_other = __shfl_xor(mm, 32, kWave), l_other = __shfl_xor(ll, 32, kWave);
+      const float m_all = fmaxf(mm, m_other);
+      const float l_all = (mm > -INFINITY ? ll * expf(mm - m_all) : 0.f) + (m_other > -INFINITY ? l_other * expf(m_other - m_all) : 0.f);
+      if (g == 0 && pair_live) {
+        red[((kWaves + wave) * kPairMax + col) * 2] = m_all;
+        red[((kWaves + wave) * kPairMax + col) * 2 + 1] = l_all;
+      }
+    }
+    __syncthreads();
+    for (int p = tid; p < pairs; p += kSplitThreads) {
+      float m_all = -INFINITY;
+      for (int w = 0; w < 2 * kWaves; ++w) m_all = fmaxf(m_all, red[(w * kPairMax + p) * 2]);
+      float l_all = 0.f;
+      for (int w = 0; w < 2 * kWaves; ++w) {
+        const float mw = red[(w * kPairMax + p) * 2];
+        if (mw > -INFINITY) l_all += red[(w * kPairMax + p) * 2 + 1] * expf(mw - m_all);
+      }
+      const int t = p / group, h = p % group;
+      const size_t at = ((size_t)(sg.row + t) * a.H + c * group + h) * a.S + split;
+      a.part_m[at] = m_all;
+      a.part_l[at] = l_all;
+    }
+    row += sg.tq;
+  }
+}
+
 // scores -> normalised weights, in place, for ALL heads of a row (every kv head's value kernel
 // mixes all of them, so each is formed once here): a block a (row, 256 entries); the shares'
 // maxima and sums of the row's heads are loaded side by side and merged in LDS first.
@@ -811,12 +969,20 @@ __global__ void pooled_merge_kernel(const float* __restrict__ part_o, T* __restr
   Elem<T>::store(out + idx, sum);
 }
 
+// whether the score kernel's matrix-core form takes these operands (bfloat16 only)
+template <typename T>
+bool scores_on_matrix_cores(const void*, const void*, const SplitArgs&) { return false; }
+template <>
+bool scores_on_matrix_cores<bf16_t>(const void* q, const void* k_cache, const SplitArgs& a) {
+  return a.dim % 16 == 0 && a.dim <= 16 * kStepsMax && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_cache % 16) == 0;
+}
+
 template <typename T>
 int launch_split(const void* q, const void* k_cache, const void* v_cache, void* out, const SplitArgs& a,
                  hipStream_t stream) {
   const int group = a.H / a.G;
   const dim3 grid((a.N + a.TQ - 1) / a.TQ, a.G, a.S);
-  const size_t lds_a = ((size_t)a.TQ * group * a.dim + (kSplitThreads / kWave) * kPairMax * 2) * 4;
+  const size_t lds_a = ((size_t)a.TQ * group * a.dim + 2 * (kSplitThreads / kWave) * kPairMax * 2) * 4;
   const size_t work = (size_t)a.TQ * group * kSplitThreads + (size_t)kStage * ((a.vdim + 3) & ~3);
   const size_t lds_b = ((size_t)group * a.H + work) * 4;
   const size_t lds_n = ((size_t)2 * a.H * a.S + 2 * a.H) * 4;
@@ -831,7 +997,18 @@ int launch_split(const void* q, const void* k_cache, const void* v_cache, void* 
     if (err != hipSuccess) return (int)err;
     allowed = true;
   }
-  pooled_scores_kernel<T><<<grid, kSplitThreads, lds_a, stream>>>((const T*)q, (const T*)k_cache, a);
+  if (scores_on_matrix_cores<T>(q, k_cache, a)) {
+    static bool mfma_allowed = false;
+    if (!mfma_allowed) {
+      const hipError_t err = hipFuncSetAttribute((const void*)pooled_scores_mfma_kernel,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (err != hipSuccess) return (int)err;
+      mfma_allowed = true;
+    }
+    pooled_scores_mfma_kernel<<<grid, kSplitThreads, lds_a, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, a);
+  } else {
+    pooled_scores_kernel<T><<<grid, kSplitThreads, lds_a, stream>>>((const T*)q, (const T*)k_cache, a);
+  }
   pooled_normalize_kernel<<<dim3(a.N, (a.Emax + kSplitThreads - 1) / kSplitThreads), kSplitThreads, lds_n, stream>>>(a);
   pooled_values_kernel<T><<<grid, kSplitThreads, lds_b, stream>>>((const T*)v_cache, (T*)out, a);
   if (a.S > 1) {

@@ -597,7 +597,7 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
 
     while rows > 1 and values_lds(rows) > POOLED_SPLIT_LDS:
         rows //= 2
-    if (values_lds(rows) > POOLED_SPLIT_LDS or 4 * (rows * group * dim + 8 * POOLED_SPLIT_PAIRS) > POOLED_SPLIT_LDS
+    if (values_lds(rows) > POOLED_SPLIT_LDS or 4 * (rows * group * dim + 16 * POOLED_SPLIT_PAIRS) > POOLED_SPLIT_LDS
             or num_heads > 4096):
         return None
     most = min(longest_context, window + rows - 1) + longest_context // pool + 1
