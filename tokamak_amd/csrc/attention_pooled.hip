@@ -622,11 +622,35 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_scores_mfma_kernel(const
       float acc[kPairMax];
 #pragma unroll
       for (int p = 0; p < kPairMax; ++p) acc[p] = 0.f;
-      for (int x = 0; x < dim; ++x) {
-        const float kx = a.k_pool[pooled_at(sg.table, entry, c * dim + x, KW, a.KE, a.page_size)];
+      const size_t first = (size_t)entry * KW + (size_t)c * dim, per_page = (size_t)a.page_size * a.KE;
+      if (per_page % 4 == 0 && first % per_page + dim <= per_page) {
+        // the mean lies in one page, on a 32-byte border (dim and KW are multiples of 16): 64 numbers asked for at once
+        const float* poolp = a.k_pool + (size_t)sg.table[first / per_page] * per_page + first % per_page;
+        for (int x0 = 0; x0 < dim; x0 += 64) {
+          float kx[64];
 #pragma unroll
-        for (int p = 0; p < kPairMax; ++p)
-          if (p < pairs) acc[p] = fmaf(qs[p * dim + x], kx, acc[p]);
+          for (int u = 0; u < 8; ++u)
+            if (x0 + 8 * u < dim) load8(poolp + x0 + 8 * u, kx + 8 * u);
+#pragma unroll
+          for (int u = 0; u < 16; ++u) {
+            if (x0 + 4 * u < dim) {
+#pragma unroll
+              for (int p = 0; p < kPairMax; ++p) {
+                if (p < pairs) {
+                  const float4 qv = *reinterpret_cast<const float4*>(qs + p * dim + x0 + 4 * u);
+                  acc[p] = fmaf(qv.x, kx[4 * u], fmaf(qv.y, kx[4 * u + 1], fmaf(qv.z, kx[4 * u + 2], fmaf(qv.w, kx[4 * u + 3], acc[p]))));
+                }
+              }
+            }
+          }
+        }
+      } else {
+        for (int x = 0; x < dim; ++x) {
+          const float kx = a.k_pool[pooled_at(sg.table, entry, c * dim + x, KW, a.KE, a.page_size)];
+#pragma unroll
+          for (int p = 0; p < kPairMax; ++p)
+            if (p < pairs) acc[p] = fmaf(qs[p * dim + x], kx, acc[p]);
+        }
       }
 #pragma unroll
       for (int p = 0; p < kPairMax; ++p) {
