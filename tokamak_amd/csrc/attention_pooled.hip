@@ -356,9 +356,9 @@ __global__ void pooled_window_attention_kernel(const T* __restrict__ q, const T*
 //   scores:  a lane an entry: its key row (or block mean) against the queries of the kv head's
 //            query heads; raw scores to memory [row][entry][head], and every (row, head)'s
 //            maximum and sum of exponentials over the share.
-//   normalize: merges the shares' statistics and turns the scores of ALL heads into normalised
-//            weights, in place (the mixing needs every head's, so each is formed once).
-//   values:  mixes the weights of its entries for its own query heads, and applies them to its
+//   normalize: merges the shares' statistics, turns the scores of ALL heads into normalised
+//            weights and mixes them, in place (each exponential and each mixed weight once).
+//   values:  applies the mixed weights of its own query heads to its
 //            kv head's values (64 entries staged in LDS at a time; a thread owns four channels of a few
 //            (row, head) pairs); float32 partial outputs.
 //   merge:   adds the shares' partial outputs.
@@ -741,18 +741,24 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_scores_mfma_kernel(const
   }
 }
 
-// scores -> normalised weights, in place, for ALL heads of a row (every kv head's value kernel
-// mixes all of them, so each is formed once here): a block a (row, 256 entries); the shares'
-// maxima and sums of the row's heads are loaded side by side and merged in LDS first.
+// scores -> normalised and MIXED weights, in place, for all heads of a row: a block a (row, 256
+// entries), a thread an entry.  The shares' maxima and sums of the row's heads are loaded side by
+// side and merged in LDS first; then w_g = exp(s_g - max_g) / sum_g for every head in registers and
+// w'_h = sum_g talk[h, g] w_g written over the scores.  Each exponential and each mixed weight is
+// formed once here, and a kv head's value kernel reads its own heads' weights only.
+constexpr int kHeadsMax = 64;
 __global__ __launch_bounds__(kSplitThreads) void pooled_normalize_kernel(SplitArgs a) {
   extern __shared__ float lds[];
   const int H = a.H, S = a.S;
-  float* sm_ = lds;                 // [H][S] maxima, then as many sums
+  const int Hp = (H + 3) & ~3;
+  float* tkk = lds;                 // [H][Hp] the mixing matrix, rows padded to four with zeros
+  float* sm_ = tkk + H * Hp;        // [H][S] maxima, then as many sums
   float* mh = sm_ + 2 * H * S;      // [H]
   float* il = mh + H;               // [H]
   const int row = blockIdx.x, tid = threadIdx.x;
   const int count = H * S;
   const size_t from = (size_t)row * count;
+  for (int i = tid; i < H * Hp; i += kSplitThreads) tkk[i] = i % Hp < H ? a.talk[(i / Hp) * H + i % Hp] : 0.f;
   for (int i = tid; i < count; i += kSplitThreads) {
     sm_[i] = a.part_m[from + i];
     sm_[count + i] = a.part_l[from + i];
@@ -780,30 +786,39 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_normalize_kernel(SplitAr
   const int e = blockIdx.y * kSplitThreads + tid;
   if (e >= E) return;
   float* sc = a.scores + ((size_t)row * a.Emax + e) * H;
-  if (H % 4 == 0) {
-    for (int h0 = 0; h0 < H; h0 += 32) {
-      float4 v[8];
+  // the entry's normalised weights of every head, in registers
+  float w[kHeadsMax];
 #pragma unroll
-      for (int y = 0; y < 8; ++y)
-        if (h0 + 4 * y < H) v[y] = *reinterpret_cast<const float4*>(sc + h0 + 4 * y);
+  for (int g4 = 0; g4 < kHeadsMax; g4 += 4) {
+    if (g4 < H) {
+      float v[4];
+      if (H % 4 == 0) {
+        const float4 f = *reinterpret_cast<const float4*>(sc + g4);
+        v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+      } else {
 #pragma unroll
-      for (int y = 0; y < 8; ++y) {
-        if (h0 + 4 * y < H) {
-          const int h = h0 + 4 * y;
-          float4 w;
-          w.x = v[y].x > -INFINITY ? expf(v[y].x - mh[h]) * il[h] : 0.f;
-          w.y = v[y].y > -INFINITY ? expf(v[y].y - mh[h + 1]) * il[h + 1] : 0.f;
-          w.z = v[y].z > -INFINITY ? expf(v[y].z - mh[h + 2]) * il[h + 2] : 0.f;
-          w.w = v[y].w > -INFINITY ? expf(v[y].w - mh[h + 3]) * il[h + 3] : 0.f;
-          *reinterpret_cast<float4*>(sc + h) = w;
-        }
+        for (int y = 0; y < 4; ++y) v[y] = g4 + y < H ? sc[g4 + y] : -INFINITY;
+      }
+#pragma unroll
+      for (int y = 0; y < 4; ++y)
+        w[g4 + y] = (g4 + y < H && v[y] > -INFINITY) ? expf(v[y] - mh[g4 + y]) * il[g4 + y] : 0.f;
+    } else {
+#pragma unroll
+      for (int y = 0; y < 4; ++y) w[g4 + y] = 0.f;
+    }
+  }
+  // mixed: w'_h = sum_g talk[h, g] w_g, written over the scores
+  for (int h = 0; h < H; ++h) {
+    const float* trow = tkk + h * Hp;
+    float acc = 0.f;
+#pragma unroll
+    for (int g4 = 0; g4 < kHeadsMax; g4 += 4) {
+      if (g4 < H) {
+        const float4 t4 = *reinterpret_cast<const float4*>(trow + g4);     // (rows padded with zeros to four)
+        acc = fmaf(t4.x, w[g4], fmaf(t4.y, w[g4 + 1], fmaf(t4.z, w[g4 + 2], fmaf(t4.w, w[g4 + 3], acc))));
       }
     }
-  } else {
-    for (int h = 0; h < H; ++h) {
-      const float v = sc[h];
-      sc[h] = v > -INFINITY ? expf(v - mh[h]) * il[h] : 0.f;
-    }
+    sc[h] = acc;
   }
 }
 
@@ -844,8 +859,7 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
   extern __shared__ float lds[];
   const int H = a.H, group = a.H / a.G, vdim = a.vdim, VW = a.G * a.vdim;
   const int c = blockIdx.y, split = blockIdx.z;
-  float* tk_ = lds;                                  // [group][H]
-  float* wm = tk_ + group * H;                       // [TQ * group][kSplitThreads] mixed weights of a chunk
+  float* wm = lds;                                   // [TQ * group][kSplitThreads] mixed weights of a chunk
   const int vdimp = (vdim + 3) & ~3, upr = vdimp / 4;   // a row padded to pieces of four channels
   float* Vs = wm + a.TQ * group * kSplitThreads;     // [kStage][vdimp] values of a stage
   const int tid = threadIdx.x;
@@ -857,7 +871,6 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
   const bool owner = 4 * cg < vdim;
   const bool vvec = vdim % 4 == 0;
   const bool pvvec = vvec && ((long)a.page_size * a.VE) % 4 == 0;
-  for (int i = tid; i < group * H; i += kSplitThreads) tk_[i] = a.talk[(size_t)(c * group + i / H) * H + i % H];
   const int row_end = min(a.N, (int)(blockIdx.x + 1) * a.TQ);
   int row = blockIdx.x * a.TQ;
   while (row < row_end) {
@@ -875,45 +888,21 @@ __global__ __launch_bounds__(kSplitThreads) void pooled_values_kernel(const T* _
       __syncthreads();            // the chunk before is applied
       if (tid < ne) {
         for (int t = 0; t < g.tq; ++t) {
-          const float* sc = a.scores + ((size_t)(g.row + t) * a.Emax + e0 + tid) * H;
-          float mixed[kGroupMax];
+          const float* sc = a.scores + ((size_t)(g.row + t) * a.Emax + e0 + tid) * H + c * group;
+          if (group % 4 == 0 && H % 4 == 0) {
 #pragma unroll
-          for (int h = 0; h < kGroupMax; ++h) mixed[h] = 0.f;
-          if (H % 4 == 0) {
-            float4 ahead[8];        // the scores of 32 heads asked for at once
-#pragma unroll
-            for (int y = 0; y < 8; ++y)
-              if (4 * y < H) ahead[y] = *reinterpret_cast<const float4*>(sc + 4 * y);
-            for (int gh = 0; gh < H; gh += 4) {
-              float4 s4;
-              if (gh < 32) {
-#pragma unroll
-                for (int y = 0; y < 8; ++y)
-                  if (gh == 4 * y) s4 = ahead[y];
-              } else {
-                s4 = *reinterpret_cast<const float4*>(sc + gh);
-              }
-              const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
-              const float* w = sv;        // (normalised weights: the kernel before has seen to that)
-#pragma unroll
-              for (int h = 0; h < kGroupMax; ++h) {
-                if (h < group) {
-                  const float4 t4 = *reinterpret_cast<const float4*>(tk_ + h * H + gh);
-                  mixed[h] = fmaf(t4.x, w[0], fmaf(t4.y, w[1], fmaf(t4.z, w[2], fmaf(t4.w, w[3], mixed[h]))));
-                }
+            for (int h = 0; h < kGroupMax; h += 4) {
+              if (h < group) {
+                const float4 f = *reinterpret_cast<const float4*>(sc + h);
+                wm[(t * group + h) * kSplitThreads + tid] = f.x;
+                wm[(t * group + h + 1) * kSplitThreads + tid] = f.y;
+                wm[(t * group + h + 2) * kSplitThreads + tid] = f.z;
+                wm[(t * group + h + 3) * kSplitThreads + tid] = f.w;
               }
             }
           } else {
-            for (int gh = 0; gh < H; ++gh) {
-              const float w = sc[gh];
-#pragma unroll
-              for (int h = 0; h < kGroupMax; ++h)
-                if (h < group) mixed[h] = fmaf(tk_[h * H + gh], w, mixed[h]);
-            }
+            for (int h = 0; h < group; ++h) wm[(t * group + h) * kSplitThreads + tid] = sc[h];
           }
-#pragma unroll
-          for (int h = 0; h < kGroupMax; ++h)
-            if (h < group) wm[(t * group + h) * kSplitThreads + tid] = mixed[h];
         }
       }
       __syncthreads();
@@ -998,7 +987,10 @@ template <typename T>
 bool scores_on_matrix_cores(const void*, const void*, const SplitArgs&) { return false; }
 template <>
 bool scores_on_matrix_cores<bf16_t>(const void* q, const void* k_cache, const SplitArgs& a) {
-  return a.dim % 16 == 0 && a.dim <= 16 * kStepsMax && ((uintptr_t)q % 16) == 0 && ((uintptr_t)k_cache % 16) == 0;
+  // (tiles of a portion's rows only: a single token's four or eight pairs fill an eighth of the 32 columns,
+  // and its few entries a block are sooner walked a lane an entry: 34 against 41 us for 8 tokens over 2,058 positions)
+  return a.TQ > 1 && a.dim % 16 == 0 && a.dim <= 16 * kStepsMax && ((uintptr_t)q % 16) == 0 &&
+         ((uintptr_t)k_cache % 16) == 0;
 }
 
 template <typename T>
@@ -1008,8 +1000,8 @@ int launch_split(const void* q, const void* k_cache, const void* v_cache, void* 
   const dim3 grid((a.N + a.TQ - 1) / a.TQ, a.G, a.S);
   const size_t lds_a = ((size_t)a.TQ * group * a.dim + 2 * (kSplitThreads / kWave) * kPairMax * 2) * 4;
   const size_t work = (size_t)a.TQ * group * kSplitThreads + (size_t)kStage * ((a.vdim + 3) & ~3);
-  const size_t lds_b = ((size_t)group * a.H + work) * 4;
-  const size_t lds_n = ((size_t)2 * a.H * a.S + 2 * a.H) * 4;
+  const size_t lds_b = work * 4;
+  const size_t lds_n = ((size_t)a.H * ((a.H + 3) & ~3) + 2 * a.H * a.S + 2 * a.H) * 4;
   if (lds_a > 150 * 1024 || lds_b > 150 * 1024 || lds_n > 64 * 1024) return -3;
   static bool allowed = false;      // (per instantiation: once per storage type)
   if (!allowed) {
@@ -1148,7 +1140,7 @@ TK_API int tk_pooled_window_attention_split(int dtype, const void* q, const void
                                             int dim, int vdim, int size, int pool, int page_size, int TQ, int S,
                                             int Emax, float scale, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (H < 1 || G < 1 || H % G || H / G > kGroupMax || dim < 1 || vdim < 1 || vdim > 256 || size < 1 ||
+  if (H < 1 || H > kHeadsMax || G < 1 || H % G || H / G > kGroupMax || dim < 1 || vdim < 1 || vdim > 256 || size < 1 ||
       pool < 1 || page_size < 1 || TQ < 1 || TQ > kTileMax || TQ * (H / G) > kPairMax || S < 1 || Emax < 1 ||
       (long)KE * pool < (long)G * dim || (long)VE * pool < (long)G * vdim)
     return -2;

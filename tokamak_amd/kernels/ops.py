@@ -574,6 +574,7 @@ POOLED_ONE_KERNEL_ONLY = False   # tests set this to run the one-kernel form on 
 POOLED_SPLIT_GROUP = 16      # query heads a kv head, value channels and rows times heads a block
 POOLED_SPLIT_VDIM = 256      # that the three-kernel form of the attention takes
 POOLED_SPLIT_PAIRS = 32
+POOLED_SPLIT_HEADS = 64      # heads whose weights a thread of the mixing kernel holds
 POOLED_SPLIT_BLOCKS = 512    # blocks wanted: two a CU run at once (some 200 registers a lane), a third waits for a whole turn
 POOLED_SPLIT_LDS = 150 * 1024
 
@@ -587,13 +588,13 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
     from tokamak_amd.kernels.attention import quarter_octave_at_least
 
     group = num_heads // num_kv_heads
-    if group > POOLED_SPLIT_GROUP or vdim > POOLED_SPLIT_VDIM or POOLED_ONE_KERNEL_ONLY:
+    if group > POOLED_SPLIT_GROUP or vdim > POOLED_SPLIT_VDIM or num_heads > POOLED_SPLIT_HEADS or POOLED_ONE_KERNEL_ONLY:
         return None
     # the length rounded as recorded steps round it: a step computes the same bits recorded or not
     longest_context = quarter_octave_at_least(longest_context, 64)
     rows = 1 if longest_span <= 1 else max(1, min(8, POOLED_SPLIT_PAIRS // group))
     def values_lds(rows: int) -> int:
-        return 4 * (group * num_heads + rows * group * 256 + 64 * (vdim + 3))
+        return 4 * (rows * group * 256 + 64 * (vdim + 3))
 
     while rows > 1 and values_lds(rows) > POOLED_SPLIT_LDS:
         rows //= 2
@@ -603,7 +604,7 @@ def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, wi
     most = min(longest_context, window + rows - 1) + longest_context // pool + 1
     blocks = -(-n // rows) * num_kv_heads
     # (a share of at least 32 entries; the shares' statistics of a row's heads fit the LDS they are merged in)
-    shares = max(1, min(32, POOLED_SPLIT_BLOCKS // blocks, -(-most // 32), 4096 // num_heads))
+    shares = max(1, min(32, POOLED_SPLIT_BLOCKS // blocks, -(-most // 32), 2048 // num_heads))
     return rows, shares, most
 
 
