@@ -1130,7 +1130,7 @@ TK_API int tk_pooled_window_attention(int dtype, const void* q, const void* k_ca
   return launch_status();
 }
 
-// The three-kernel form.  scores [N, Emax, H], part_m / part_l [N, H, S], part_o [S, N, H * vdim]
+// The four-kernel form.  scores [N, Emax, H], part_m / part_l [N, H, S], part_o [S, N, H * vdim]
 // (unused if S == 1) are float32 scratch; Emax bounds the entries any tile of TQ rows sees.
 TK_API int tk_pooled_window_attention_split(int dtype, const void* q, const void* k_cache, const void* v_cache,
                                             const float* k_pool, const float* v_pool, int KE, int VE, void* out,

@@ -572,7 +572,7 @@ def pooled_window_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, l
 POOLED_ONE_KERNEL_ONLY = False   # tests set this to run the one-kernel form on sizes the other form takes
 
 POOLED_SPLIT_GROUP = 16      # query heads a kv head, value channels and rows times heads a block
-POOLED_SPLIT_VDIM = 256      # that the three-kernel form of the attention takes
+POOLED_SPLIT_VDIM = 256      # that the four-kernel form of the attention takes
 POOLED_SPLIT_PAIRS = 32
 POOLED_SPLIT_HEADS = 64      # heads whose weights a thread of the mixing kernel holds
 POOLED_SPLIT_BLOCKS = 512    # blocks wanted: two a CU run at once (some 200 registers a lane), a third waits for a whole turn
@@ -581,7 +581,7 @@ POOLED_SPLIT_LDS = 150 * 1024
 
 def pooled_split_plan(num_heads: int, num_kv_heads: int, dim: int, vdim: int, window: int, pool: int, n: int,
                       longest_span: int, longest_context: int) -> tuple[int, int, int] | None:
-    """(rows a block, shares of the entries, most entries a tile sees) for the three-kernel form of
+    """(rows a block, shares of the entries, most entries a tile sees) for the four-kernel form of
     the pooled-window attention, or None where its sizes do not fit and the one-kernel form runs.
     Up to 8 consecutive rows of a portion share the rows a lane loads; single tokens take a
     block each; the entries are cut in shares until about a thousand blocks exist."""
