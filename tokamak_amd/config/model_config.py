@@ -100,11 +100,15 @@ class LayerCall:
     holds several mixers brings a tuple of slots, one for each mixer in the order
     the layer names them.  A call with ``writes_cache=False`` only reads its slots
     (it attends over keys and values another call stored) and stores nothing itself.
+    ``adds_embedding``: before the call the embedding's output for the step's tokens is
+    added to the residual stream once more (a model that runs a stretch of layers several
+    times and feeds its input in again at the start of each further pass).
     """
 
     layer: int
     cache: int | tuple[int, ...]
     writes_cache: bool = True
+    adds_embedding: bool = False
 
     @property
     def slots(self) -> tuple[int, ...]:

@@ -15,7 +15,11 @@
 // depend on how the request was cut into steps, on what else is in the batch, or on
 // whether the token ran alone or in a tile (equal bits).
 //
-// Cache pages: K [nkv][hd/8][ps][8], V [nkv][hd/16][ps/4][16][4] (see elementwise.hip).
+// Keys and values may differ in size (hd and vd).  What a query sees besides causality is given
+// by `span`: 0 everything before it, W > 0 the last W positions, -C < 0 the positions of its own
+// chunk of C (chunks counted from position 0 of the sequence).
+//
+// Cache pages: K [nkv][hd/8][ps][8], V [nkv][vd/16][ps/4][16][4] (see elementwise.hip).
 #include "common.h"
 #include "slots.h"
 
@@ -66,13 +70,13 @@ struct GenericItems {
 
 // QT: queries of a block; HEADS: they are heads of one group at one token (blockIdx.y is the kv
 // head, blockIdx.z the piece of the group), else tokens of one tile at one head (blockIdx.y).
-// SLOTS: dimensions a lane owns (hd <= 64 * SLOTS).
+// SLOTS: value dimensions a lane owns (vd <= 64 * SLOTS).
 template <typename T, int QT, bool HEADS, int SLOTS>
 __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, GenericItems items, T* __restrict__ out, int nh, int nkv,
-    int hd, int ps, int max_pages, float scale, int window) {
+    int hd, int vd, int ps, int max_pages, float scale, int span) {
   __shared__ __attribute__((aligned(16))) float q_s[QT][kMaxHd];
   __shared__ __attribute__((aligned(16))) float p_s[kWaves][kWave][QT];
   __shared__ long base_s[kWaves][kWave];  // where a key's values lie (a quad's, for tokens that run alone), or -1
@@ -104,11 +108,11 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     const int u = min(t, cnt - 1);
     row[t] = HEADS ? (size_t)n0 * nh + head0 + u : (size_t)(n0 + u) * nh + head0;
     pos[t] = positions[HEADS ? n0 : n0 + u];
-    first[t] = (window > 0 && pos[t] - window + 1 > 0) ? pos[t] - window + 1 : 0;
+    first[t] = span > 0 ? (pos[t] - span + 1 > 0 ? pos[t] - span + 1 : 0) : span < 0 ? pos[t] - pos[t] % (-span) : 0;
   }
   const int lo = first[0], hi = pos[QT - 1];  // positions ascend within a tile
-  const size_t page_elems = (size_t)nkv * hd * ps;
-  const size_t head_off = (size_t)kvh * hd * ps;
+  const size_t page_elems = (size_t)nkv * hd * ps, v_page_elems = (size_t)nkv * vd * ps;
+  const size_t head_off = (size_t)kvh * hd * ps, v_head_off = (size_t)kvh * vd * ps;
 
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
@@ -143,7 +147,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     if (BATCHED && (lane & 3) == 0 && c <= hi && c + 3 >= lo) {
       // the values of four consecutive keys of a dimension are one piece of a page
       const int page = table[c / ps];
-      vbase = (long)((size_t)page * page_elems + head_off + (size_t)((c % ps) >> 2) * 64);
+      vbase = (long)((size_t)page * v_page_elems + v_head_off + (size_t)((c % ps) >> 2) * 64);
     }
     if (loaded) {
       const int page = table[c / ps];
@@ -179,7 +183,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
             for (int e = 0; e < 8; ++e) dot[t] = fmaf(q_s[t][j * 8 + e], k8[e], dot[t]);
           }
         }
-        vbase = (long)((size_t)page * page_elems + head_off + (size_t)(off >> 2) * 64 + (off & 3));
+        vbase = (long)((size_t)page * v_page_elems + v_head_off + (size_t)(off >> 2) * 64 + (off & 3));
       }
     }
     float alpha[QT], p[QT];
@@ -209,7 +213,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
 #pragma unroll
     for (int i = 0; i < SLOTS; ++i) {
       const int d = lane + i * kWave;
-      if (d < hd) {
+      if (d < vd) {
         const size_t v_dim_off = (size_t)(d >> 4) * (ps >> 2) * 64 + (d & 15) * 4;
         float a[QT];
 #pragma unroll
@@ -267,10 +271,10 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
 #pragma unroll
     for (int i = 0; i < SLOTS; ++i) {
       const int d = lane + i * kWave;
-      if (d < hd) acc_s[wave][d] = acc[i][t];
+      if (d < vd) acc_s[wave][d] = acc[i][t];
     }
     __syncthreads();
-    if (tid < hd) {
+    if (tid < vd) {
       float top = m_s[0];
 #pragma unroll
       for (int w = 1; w < kWaves; ++w) top = fmaxf(top, m_s[w]);
@@ -281,7 +285,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
         sum = fmaf(l_s[w], e, sum);
         o = fmaf(acc_s[w][tid], e, o);
       }
-      Elem<T>::store(out + row[t] * hd + tid, o / sum);
+      Elem<T>::store(out + row[t] * vd + tid, o / sum);
     }
   }
 }
@@ -289,14 +293,14 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
 template <typename T, int SLOTS>
 static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const int* block_tables,
                            const int* positions, const int* req_of_token, GenericItems items,
-                           int num_single, int num_tiles, T* out, int nh, int nkv, int hd, int ps,
-                           int max_pages, float scale, int window, int share_heads, hipStream_t stream) {
+                           int num_single, int num_tiles, T* out, int nh, int nkv, int hd, int vd, int ps,
+                           int max_pages, float scale, int span, int share_heads, hipStream_t stream) {
   const int group = nh / nkv;
 #define TK_ALONE(QT_)                                                                               \
   paged_attention_generic_kernel<T, QT_, true, SLOTS>                                               \
       <<<dim3(num_single, nkv, (group + QT_ - 1) / QT_), kWaves * kWave, 0, stream>>>(              \
-          q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,  \
-          max_pages, scale, window)
+          q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, vd,  \
+          ps, max_pages, scale, span)
   if (num_single > 0) {
     // the heads of a group share a block if that still gives every CU one (the result is the
     // same either way): at batch 64 of an 8B-shaped layer a third faster, at batch 8 slower
@@ -311,8 +315,8 @@ static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const
   if (num_tiles > 0)
     paged_attention_generic_kernel<T, kQueries, false, SLOTS>
         <<<dim3(num_tiles, nh, kTileTokens / kQueries), kWaves * kWave, 0, stream>>>(
-            q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,
-            max_pages, scale, window);
+            q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, vd, ps,
+            max_pages, scale, span);
 }
 
 // tile_first / tile_count (num_tiles of them) and single (num_single token rows): the step's work
@@ -322,12 +326,12 @@ static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const
 TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_cache,
                                       const void* v_cache, const int* block_tables,
                                       const int* positions, const int* req_of_token, void* out,
-                                      int N, int nh, int nkv, int hd, int ps, int max_pages,
-                                      float scale, int window, const int* tile_first,
+                                      int N, int nh, int nkv, int hd, int vd, int ps, int max_pages,
+                                      float scale, int span, const int* tile_first,
                                       const int* tile_count, int num_tiles, const int* single,
                                       int num_single, int share_heads, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (hd > kMaxHd || hd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
+  if (hd > kMaxHd || hd % 8 != 0 || vd > kMaxHd || vd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
   if (tile_first == nullptr) {
     num_tiles = 0;
     single = nullptr;
@@ -339,14 +343,14 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
 #define TK_GENERIC(T_, SLOTS_)                                                                      \
   launch_generic<T_, SLOTS_>((const T_*)q, (const T_*)k_cache, (const T_*)v_cache, block_tables,    \
                              positions, req_of_token, items, num_single, num_tiles, (T_*)out, nh,   \
-                             nkv, hd, ps, max_pages, scale, window, share_heads, stream)
+                             nkv, hd, vd, ps, max_pages, scale, span, share_heads, stream)
   if (dtype == 0) {
-    if (hd <= 128) TK_GENERIC(float, 2);
-    else if (hd <= 256) TK_GENERIC(float, 4);
+    if (vd <= 128) TK_GENERIC(float, 2);
+    else if (vd <= 256) TK_GENERIC(float, 4);
     else TK_GENERIC(float, 8);
   } else {
-    if (hd <= 128) TK_GENERIC(bf16_t, 2);
-    else if (hd <= 256) TK_GENERIC(bf16_t, 4);
+    if (vd <= 128) TK_GENERIC(bf16_t, 2);
+    else if (vd <= 256) TK_GENERIC(bf16_t, 4);
     else TK_GENERIC(bf16_t, 8);
   }
 #undef TK_GENERIC

@@ -8,11 +8,13 @@
 using namespace tk;
 
 // ---------------------------------------------------------------------------
-// embedding: resid[n, :] = float(table[ids[n], :]); an id outside [0, V) gives NaN
+// embedding: resid[n, :] = float(table[ids[n], :]) * scale, or with `accumulate`
+// resid[n, :] += float(table[ids[n], :]) * scale (the same rows added to the stream once
+// more, for a model that feeds its input in again); an id outside [0, V) gives NaN
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ resid, int H, int V) {
+                                    float* __restrict__ resid, int H, int V, float scale, int accumulate) {
   const int n = blockIdx.x;
   const int id = ids[n];
   float* out = resid + (size_t)n * H;
@@ -21,16 +23,20 @@ __global__ void embed_gather_kernel(const T* __restrict__ table, const int* __re
     return;
   }
   const T* row = table + (size_t)id * H;
-  for (int d = threadIdx.x; d < H; d += blockDim.x) out[d] = Elem<T>::load(row + d);
+  if (accumulate) {
+    for (int d = threadIdx.x; d < H; d += blockDim.x) out[d] += Elem<T>::load(row + d) * scale;
+  } else {
+    for (int d = threadIdx.x; d < H; d += blockDim.x) out[d] = Elem<T>::load(row + d) * scale;
+  }
 }
 
 TK_API int tk_embed_gather(int dtype, const void* table, const int* ids, float* resid, int N, int H,
-                           int V, hipStream_t stream) {
+                           int V, float scale, int accumulate, hipStream_t stream) {
   if (N <= 0) return 0;
   if (dtype == 0)
-    embed_gather_kernel<float><<<N, 256, 0, stream>>>((const float*)table, ids, resid, H, V);
+    embed_gather_kernel<float><<<N, 256, 0, stream>>>((const float*)table, ids, resid, H, V, scale, accumulate);
   else
-    embed_gather_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)table, ids, resid, H, V);
+    embed_gather_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)table, ids, resid, H, V, scale, accumulate);
   return launch_status();
 }
 
@@ -663,9 +669,138 @@ TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long 
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// Half-split rotation of the first `rot` dims of q and k, THEN each head of q and k divided by
+// its root mean square over all hd dims (times a weight per dim, if one is given), q written
+// out, k and v written into the paged cache.  Keys and values may differ in size:
+// qkv: [N, nh * hd + nkv_in * hd + nkv_in * vd] (q heads, k heads, v heads); with nkv_in == 0
+// the input holds q heads only and nothing is stored.  Cache pages as above, the value page
+// with vd in place of hd: K page [nkv][hd/8][ps][8], V page [nkv][vd/16][ps/4][16][4].
+// One wave per (token, head), four waves a block, each with an LDS row of its own.
+// ---------------------------------------------------------------------------
+template <typename T, typename TIN>
+__global__ void rope_norm_store_kernel(
+    const TIN* __restrict__ qkv, int parts, long part_stride, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ block_tables, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, int nh, int nkv_in, int nkv, int hd, int vd, int rot, int ps, int max_pages,
+    int unit, float eps, int num_pairs) {
+  __shared__ float vecs[kPairsPerBlock][kMaxHeadDim];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int heads = nh + 2 * nkv_in;
+  const int pair = blockIdx.x * kPairsPerBlock + wave;
+  if (pair >= num_pairs) return;  // nothing below synchronises across waves
+  const int n = pair / heads, head = pair - n * heads;
+  float* vec = vecs[wave];
+  const size_t row_width = (size_t)(nh + nkv_in) * hd + (size_t)nkv_in * vd;
+  const bool is_q = head < nh;
+  const bool is_k = !is_q && head < nh + nkv_in;
+  const int width = (is_q || is_k) ? hd : vd;
+  const size_t head_at = (is_q || is_k) ? (size_t)head * hd : (size_t)(nh + nkv_in) * hd + (size_t)(head - nh - nkv_in) * vd;
+  const TIN* src = qkv + (size_t)n * row_width + head_at;
+  for (int d = lane; d < width; d += kWave) {
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += Elem<TIN>::load(src + (size_t)p * part_stride + d);
+    vec[d] = v;
+  }
+  wave_lds_sync();
+  if (is_q || is_k) {
+    const int half = rot / 2;
+    float lo[kMaxHeadDim / 2 / kWave], hi[kMaxHeadDim / 2 / kWave];
+    int cnt = 0;
+    for (int j = lane; j < half; j += kWave, ++cnt) {
+      const float c = cos_t[(size_t)n * half + j], s = sin_t[(size_t)n * half + j];
+      const float a = vec[j], b = vec[j + half];
+      lo[cnt] = a * c - b * s;
+      hi[cnt] = b * c + a * s;
+    }
+    wave_lds_sync();
+    cnt = 0;
+    for (int j = lane; j < half; j += kWave, ++cnt) {
+      vec[j] = lo[cnt];
+      vec[j + half] = hi[cnt];
+    }
+    wave_lds_sync();
+    if (unit) {
+      float ss = 0.f;
+      for (int d = lane; d < hd; d += kWave) ss += vec[d] * vec[d];
+      ss = wave_sum(ss);
+      const float rstd = 1.f / sqrtf(ss / (float)hd + eps);
+      const float* w = is_q ? q_weight : k_weight;
+      for (int d = lane; d < hd; d += kWave) vec[d] = vec[d] * rstd * (w ? w[d] : 1.f);   // (a lane rewrites what it read)
+      wave_lds_sync();
+    }
+  }
+  if (is_q) {
+    T* dst = q_out + ((size_t)n * nh + head) * hd;
+    for (int d = lane; d < hd; d += kWave) Elem<T>::store(dst + d, vec[d]);
+    return;
+  }
+  const int pos = positions[n];
+  const int page = block_tables[(size_t)req_of_token[n] * max_pages + pos / ps];
+  const int off = pos % ps;
+  if (is_k) {
+    const int kvh = head - nh;
+    T* base = k_cache + (size_t)page * ((size_t)nkv * hd * ps) + (size_t)kvh * hd * ps;
+    for (int d = lane; d < hd; d += kWave)
+      Elem<T>::store(base + ((size_t)(d >> 3) * ps + off) * 8 + (d & 7), vec[d]);
+  } else {
+    const int kvh = head - nh - nkv_in;
+    T* base = v_cache + (size_t)page * ((size_t)nkv * vd * ps) + (size_t)kvh * vd * ps;
+    for (int d = lane; d < vd; d += kWave)
+      Elem<T>::store(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3), vec[d]);
+  }
+}
+
+// in_f32: qkv is float32 (possibly `parts` partial sums, part_stride elements apart)
+TK_API int tk_rope_norm_store(int dtype, const void* qkv, int in_f32, int parts, long part_stride,
+                              const float* q_weight, const float* k_weight, const float* cos_t,
+                              const float* sin_t, const int* positions, const int* req_of_token,
+                              const int* block_tables, void* q_out, void* k_cache, void* v_cache,
+                              int N, int nh, int nkv_in, int nkv, int hd, int vd, int rot, int ps,
+                              int max_pages, int unit, float eps, hipStream_t stream) {
+  if (N <= 0) return 0;
+  if (hd > kMaxHeadDim || vd > kMaxHeadDim || hd % 8 != 0 || vd % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0) return -1;
+  if (nkv_in != 0 && nkv_in != nkv) return -1;
+  if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
+  const long pairs = (long)N * (nh + 2 * nkv_in);
+  if (pairs > 0x7fffffffL) return -1;
+  const unsigned grid = (unsigned)((pairs + kPairsPerBlock - 1) / kPairsPerBlock);
+#define TK_RN(T_, TIN_)                                                                          \
+  rope_norm_store_kernel<T_, TIN_><<<grid, kWave * kPairsPerBlock, 0, stream>>>(                 \
+      (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,         \
+      req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, hd,   \
+      vd, rot, ps, max_pages, unit, eps, (int)pairs)
+  if (dtype == 0) TK_RN(float, float);
+  else if (in_f32) TK_RN(bf16_t, float);
+  else TK_RN(bf16_t, bf16_t);
+#undef TK_RN
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// logits in place: x <- x * scale, then (cap > 0) x <- cap * tanh(x / cap)
+// ---------------------------------------------------------------------------
+__global__ void scale_softcap_kernel(float* __restrict__ x, size_t total, float scale, float cap) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float v = x[idx] * scale;
+  if (cap > 0.f) v = cap * tanhf(v / cap);
+  x[idx] = v;
+}
+
+TK_API int tk_scale_softcap(float* x, long total, float scale, float cap, hipStream_t stream) {
+  if (total <= 0) return 0;
+  scale_softcap_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(x, (size_t)total, scale, cap);
+  return launch_status();
+}
+
 // the same entry points in slot form (slots.h), for launch lists
 TK_SLOTS(tk_add_rmsnorm)
 TK_SLOTS(tk_rope_tables)
 TK_SLOTS(tk_qknorm_rope_store)
 TK_SLOTS(tk_silu_mul)
 TK_SLOTS(tk_scaled_sum)
+TK_SLOTS(tk_rope_norm_store)
+TK_SLOTS(tk_scale_softcap)

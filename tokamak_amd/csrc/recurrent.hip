@@ -9,6 +9,11 @@
 //   over the step's tokens in order, the state S [dim, dim] in float32 registers (a thread owns a
 //   few key channels of a column), followed by the head's unit norm, a gain and a SiLU gate.
 //
+// gla_scan: per (request, head) the gated linear attention recurrence
+//     S <- diag(a_t) S + k_t v_t^T ;  o_t = S^T (q_t * q_scale) ,  a_t = sigmoid(z_t + b)^(1/tau)
+//   with a state S [dim, vdim] whose two sides may differ, the newest token already in S when it
+//   is read, followed by the head's unit norm, a gain per value channel and a SiLU gate.
+//
 // Decays, exponentials, the state and the norm are float32 whatever the storage type.
 #include "common.h"
 #include "slots.h"
@@ -305,6 +310,160 @@ int launch_scan(ScanIn r, ScanIn k, ScanIn v, ScanIn g, ScanIn d, const float* w
   return launch_status();
 }
 
+struct GlaShape {
+  int heads, dim, vdim, columns, slices, slice;   // threads = columns * slices; a thread owns `slice` key channels of a value column
+};
+
+// A block a (request, head).  Thread (ks, j) owns rows [ks * slice, (ks + 1) * slice) of column j
+// (a value channel) of the state in registers; the groups' partial outputs meet in LDS.  Tokens
+// run in order, eight staged at a time.  a = sigmoid(z)^(1/tau) is formed as
+// exp(-softplus(-z) / tau), softplus(x) = max(x, 0) + log1p(exp(-|x|)).
+template <typename T, int SLICE, bool PLAIN>
+__global__ __launch_bounds__(1024) void gla_scan_kernel(
+    ScanIn q_in, ScanIn k_in, ScanIn v_in, ScanIn g_in, ScanIn z_in, const float* __restrict__ bias,
+    const float* __restrict__ gain, float* __restrict__ state, const int* __restrict__ q_start,
+    const int* __restrict__ state_slots, T* __restrict__ out, GlaShape sh, float q_scale, float inv_tau, float eps) {
+  constexpr int TB = kScanTokens;
+  extern __shared__ float lds[];
+  const int dim = sh.dim, vdim = sh.vdim, CT = sh.columns, KS = sh.slices, slice = sh.slice;
+  const int dimp = (dim + 3) & ~3, vdimp = (vdim + 3) & ~3;
+  float* qq = lds;                     // [TB][dimp] each
+  float* kk = qq + TB * dimp;
+  float* aa = kk + TB * dimp;
+  float* os = aa + TB * dimp;          // [TB][vdimp]
+  float* rstd = os + TB * vdimp;       // [TB]
+  float* part = rstd + TB;             // [KS][TB][CT]
+  const int req = blockIdx.x, head = blockIdx.y;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int ks = tid / CT, j = tid - ks * CT;
+  const bool live = j < vdim;
+  const int k0 = ks * slice;
+  const int kn = max(0, min(slice, dim - k0));     // key channels of this thread's slice that exist
+  const int KW = sh.heads * dim, VW = sh.heads * vdim;
+  const int kbase = head * dim, vbase = head * vdim;
+  const int first = q_start[req], end = q_start[req + 1];
+  float* S = state + ((size_t)state_slots[req] * sh.heads + head) * dim * vdim;
+  float s[SLICE];
+#pragma unroll
+  for (int x = 0; x < SLICE; ++x) s[x] = (live && x < kn) ? S[(size_t)(k0 + x) * vdim + j] : 0.f;
+  const float gj = live ? gain[j] : 0.f;
+  const int lane = tid & (kWave - 1), wave = tid / kWave, nwaves = nthreads / kWave;
+
+  for (int t0 = first; t0 < end; t0 += TB) {
+    const int tb = min(TB, end - t0);
+    for (int i = tid; i < tb * dim; i += nthreads) {
+      const int t = i / dim, c = i - t * dim;
+      const size_t at = (size_t)(t0 + t) * KW + kbase + c;
+      qq[t * dimp + c] = scan_load<T, PLAIN>(q_in, at) * q_scale;
+      kk[t * dimp + c] = scan_load<T, PLAIN>(k_in, at);
+      const float x = -(scan_load<T, false>(z_in, at) + bias[kbase + c]);
+      aa[t * dimp + c] = expf(-(fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)))) * inv_tau);
+    }
+    float vloc[TB];
+#pragma unroll
+    for (int t = 0; t < TB; ++t)
+      vloc[t] = (t < tb && live) ? scan_load<T, PLAIN>(v_in, (size_t)(t0 + t) * VW + vbase + j) : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
+      if (t < tb) {
+        const float vj = vloc[t];
+        float o = 0.f;
+#pragma unroll
+        for (int x = 0; x < SLICE; x += 4) {
+          if (x < kn) {
+            const int at = t * dimp + k0 + x;       // (k0 and dimp are multiples of four)
+            const float4 q4 = *reinterpret_cast<const float4*>(qq + at);
+            const float4 k4 = *reinterpret_cast<const float4*>(kk + at);
+            const float4 a4 = *reinterpret_cast<const float4*>(aa + at);
+            const float qv[4] = {q4.x, q4.y, q4.z, q4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w};
+            const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+            for (int y = 0; y < 4; ++y) {
+              if (x + y < kn) {
+                s[x + y] = fmaf(av[y], s[x + y], kv[y] * vj);
+                o = fmaf(qv[y], s[x + y], o);
+              }
+            }
+          }
+        }
+        part[(ks * TB + t) * CT + j] = o;
+      }
+    }
+    __syncthreads();
+    for (int t = ks; t < tb; t += KS) {
+      float o = 0.f;
+      for (int q = 0; q < KS; ++q) o += part[(q * TB + t) * CT + j];
+      if (live) os[t * vdimp + j] = o;
+    }
+    __syncthreads();
+    for (int t = wave; t < tb; t += nwaves) {
+      float q = 0.f;
+      for (int x = lane; x < vdim; x += kWave) q += os[t * vdimp + x] * os[t * vdimp + x];
+      q = wave_sum(q);
+      if (lane == 0) rstd[t] = 1.f / sqrtf(q / (float)vdim + eps);
+    }
+    __syncthreads();
+    for (int t = ks; t < tb; t += KS) {
+      if (live) {
+        const size_t at = (size_t)(t0 + t) * VW + vbase + j;
+        const float g = scan_load<T, PLAIN>(g_in, at);
+        Elem<T>::store(out + at, os[t * vdimp + j] * rstd[t] * gj * (g / (1.f + expf(-g))));
+      }
+    }
+    // (the next round's staging writes qq, kk, aa, which nobody reads after the second barrier;
+    // os, rstd and part are written again only behind the next round's barriers)
+  }
+  if (live) {
+#pragma unroll
+    for (int x = 0; x < SLICE; ++x)
+      if (x < kn) S[(size_t)(k0 + x) * vdim + j] = s[x];
+  }
+}
+
+template <typename T>
+int launch_gla(ScanIn q, ScanIn k, ScanIn v, ScanIn g, ScanIn z, const float* bias, const float* gain, float* state,
+               const int* q_start, const int* state_slots, void* out, int R, int heads, int dim, int vdim,
+               float q_scale, float inv_tau, float eps, hipStream_t stream) {
+  GlaShape sh;
+  sh.heads = heads;
+  sh.dim = dim;
+  sh.vdim = vdim;
+  sh.columns = (vdim + kWave - 1) / kWave * kWave;
+  const int most = min(16, 1024 / sh.columns);                      // groups of threads that can share a head
+  sh.slice = max(4, ((dim + most - 1) / most + 3) / 4 * 4);
+  sh.slices = (dim + sh.slice - 1) / sh.slice;
+  const int threads = sh.columns * sh.slices;
+  const int dimp = (dim + 3) & ~3, vdimp = (vdim + 3) & ~3;
+  const size_t lds = ((size_t)3 * kScanTokens * dimp + (size_t)kScanTokens * vdimp + kScanTokens +
+                      (size_t)sh.slices * kScanTokens * sh.columns) * 4;
+  const dim3 grid(R, heads);
+  const bool plain = !q.f32 && !k.f32 && !v.f32 && !g.f32;
+#define TK_GLA_AS(SLICE, PLAIN)                                                                               \
+  {                                                                                                           \
+    static bool allowed = false;                                                                              \
+    if (!allowed) {                                                                                           \
+      const hipError_t err = hipFuncSetAttribute((const void*)gla_scan_kernel<T, SLICE, PLAIN>,               \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);     \
+      if (err != hipSuccess) return (int)err;                                                                 \
+      allowed = true;                                                                                         \
+    }                                                                                                         \
+    gla_scan_kernel<T, SLICE, PLAIN><<<grid, threads, lds, stream>>>(q, k, v, g, z, bias, gain, state, q_start, \
+                                                                     state_slots, (T*)out, sh, q_scale, inv_tau, eps); \
+  }
+#define TK_GLA(SLICE)                 \
+  {                                   \
+    if (plain) TK_GLA_AS(SLICE, true) \
+    else TK_GLA_AS(SLICE, false)      \
+  }
+  if (sh.slice <= 4) TK_GLA(4)
+  else if (sh.slice <= 16) TK_GLA(16)
+  else TK_GLA(64)
+#undef TK_GLA_AS
+#undef TK_GLA
+  return launch_status();
+}
+
 }  // namespace
 
 // out[s][n] = h[n] + (prev(n) - h[n]) * mu[s]; `last` [slots, W] float32 holds each request's
@@ -368,6 +527,27 @@ TK_API int tk_wkv_scan(int dtype, const void* r, int r_f32, int r_parts, long r_
                              stream);
 }
 
+// q, k, z (the decay's pre-activation, to which `bias` is added): [N, heads * dim]; v, g (gate):
+// [N, heads * vdim]; each in dtype, or float32, or float32 partial sums [parts, N, width]; out
+// [N, heads * vdim] in dtype; state [slots, heads, dim, vdim] float32.  dim, vdim <= 256.
+TK_API int tk_gla_scan(int dtype, const void* q, int q_f32, int q_parts, long q_stride, const void* k, int k_f32,
+                       int k_parts, long k_stride, const void* v, int v_f32, int v_parts, long v_stride,
+                       const void* g, int g_f32, int g_parts, long g_stride, const void* z, int z_f32, int z_parts,
+                       long z_stride, const float* bias, const float* gain, float* state, const int* q_start,
+                       const int* state_slots, void* out, int R, int heads, int dim, int vdim, float q_scale,
+                       float inv_tau, float eps, hipStream_t stream) {
+  if (R <= 0 || heads <= 0) return 0;
+  if (dim < 1 || dim > 256 || vdim < 1 || vdim > 256) return -2;
+  const ScanIn qi{q, q_f32, q_parts, q_stride}, ki{k, k_f32, k_parts, k_stride}, vi{v, v_f32, v_parts, v_stride},
+      gi{g, g_f32, g_parts, g_stride}, zi{z, z_f32, z_parts, z_stride};
+  if (dtype == 0)
+    return launch_gla<float>(qi, ki, vi, gi, zi, bias, gain, state, q_start, state_slots, out, R, heads, dim, vdim,
+                             q_scale, inv_tau, eps, stream);
+  return launch_gla<bf16_t>(qi, ki, vi, gi, zi, bias, gain, state, q_start, state_slots, out, R, heads, dim, vdim,
+                            q_scale, inv_tau, eps, stream);
+}
+
 TK_SLOTS(tk_token_shift)
 TK_SLOTS(tk_tanh)
 TK_SLOTS(tk_wkv_scan)
+TK_SLOTS(tk_gla_scan)

@@ -186,6 +186,10 @@ class LayeredModel:
         for at, call in enumerate(order):
             block = self.blocks[call.layer]
             store = self._store_of(call, storage)
+            if call.adds_embedding:
+                if isinstance(pending, Added):
+                    pending = None      # (what the last product prepared for the next norm no longer holds)
+                self.embedding.add_to(batch, resid)
             kwargs = {}
             if block.fuses_residual:
                 # the norm that reads the stream after this block: its last product may prepare for it

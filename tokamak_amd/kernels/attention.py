@@ -273,7 +273,7 @@ def decode_attention_fused(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, 
 
 
 def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads, num_kv_heads,
-                    head_dim, page_size, scale, window=None) -> None:
+                    head_dim, page_size, scale, window=None, value_dim=None, chunk=None) -> None:
     """out[n] = softmax(q[n] . K[0..pos_n] * scale) V, per head, over the pages
     of each token's request.
 
@@ -284,7 +284,10 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     a thousand keys or more; tiles of 16 otherwise, their keys split over blocks
     when the tiles are few and the context long.  Everything else, and whatever
     the MFMA library does not instantiate: the generic float32-arithmetic kernel.
+    ``value_dim``: size of a value head if not ``head_dim``.  ``chunk``: a query sees the
+    keys of its own chunk of that many positions only (the generic kernel).
     """
+    value_dim = head_dim if value_dim is None else value_dim
     work = work_of(batch)
     profiling = ops._profile is not None
     if profiling:
@@ -292,9 +295,14 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
         decode_keys = sum(c + 1 for c, n in zip(batch.ctx_lens, batch.q_lens) if n == 1)
         tile_pairs = sum(n * c + n * (n + 1) // 2 for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
         tile_keys = sum(c + n for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
-        kv_token_bytes = 2 * num_kv_heads * head_dim * q.element_size()
-        flops_per_pair = 4.0 * num_heads * head_dim
-    if mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
+        if chunk:
+            # a query at position p sees p % chunk + 1 keys
+            decode_keys = sum(c % chunk + 1 for c, n in zip(batch.ctx_lens, batch.q_lens) if n == 1)
+            tile_pairs = sum(sum((c + i) % chunk + 1 for i in range(n)) for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+            tile_keys = sum(n + c % chunk for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+        kv_token_bytes = num_kv_heads * (head_dim + value_dim) * q.element_size()
+        flops_per_pair = 2.0 * num_heads * (head_dim + value_dim)
+    if not chunk and value_dim == head_dim and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
         if _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, num_heads=num_heads,
                                  num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale,
                                  note=(decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair) if profiling else None):
@@ -305,7 +313,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-        scale=scale, window=window,
+        scale=scale, window=window, value_dim=value_dim, chunk=chunk,
         tiles=(work.tile_first, work.tile_count, work.num_tiles, work.single, work.num_single))
 
 

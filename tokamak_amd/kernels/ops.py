@@ -166,7 +166,7 @@ def _check(status: int, name: str) -> None:
 
 _SIGS = {
     "elementwise": {
-        "tk_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "tk_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
         "tk_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p,
                            c_void_p, c_int, c_int, c_float, c_int, c_void_p],
@@ -174,6 +174,10 @@ _SIGS = {
         "tk_qknorm_rope_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+        "tk_rope_norm_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+        "tk_scale_softcap": [c_void_p, c_long, c_float, c_float, c_void_p],
         "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "tk_scaled_sum": [c_int, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float,
                           c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -203,6 +207,15 @@ _SIGS = {
                         c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p,
                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
                         c_void_p],
+        "tk_gla_scan": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int,
+                        c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_long, c_void_p,
+                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
+                        c_float, c_void_p],
+    },
+    "moe": {
+        "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_moe_gate_up": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_moe_down": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     },
     "gemm_tiled": {
         "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
@@ -231,7 +244,7 @@ _SIGS = {
     },
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                        c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     },
     "attention_mfma": {
@@ -337,8 +350,10 @@ def _fn(library: str, name: str):
 
 
 # ---------------------------------------------------------------------------
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor) -> None:
-    """resid[n] = float(table[ids[n]]); resid is float32 [N, H]."""
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor, scale: float = 1.0,
+                 accumulate: bool = False) -> None:
+    """resid[n] = float(table[ids[n]]) * scale (``accumulate``: added to what resid[n] holds);
+    resid is float32 [N, H]."""
     _gpu(table, ids, resid)
     n = ids.numel()
     v, h = table.shape
@@ -347,7 +362,8 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor) ->
           "residual buffer must be float32 [>=N, H]")
     _note(f"{n}x{h}", n * h * (table.element_size() + 4))
     _check(_fn("elementwise", "tk_embed_gather")(_code(table.dtype), _p(table), _p(ids), _p(resid),
-                                                 n, h, v, _stream()), "embed_gather")
+                                                 n, h, v, float(scale), int(bool(accumulate)), _stream()),
+           "embed_gather")
 
 
 def feed_tokens(ids: torch.Tensor, sampled: torch.Tensor, slots: torch.Tensor, rows: torch.Tensor, count: int,
@@ -449,6 +465,54 @@ def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
         _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
         nkv_in, num_kv_heads, head_dim, rotary_dim, page_size, max_pages, float(eps), _stream()),
         "qknorm_rope_store")
+
+
+def rope_norm_store(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None,
+                    cos: torch.Tensor | None, sin: torch.Tensor | None, positions: torch.Tensor,
+                    req_of_token: torch.Tensor, block_tables: torch.Tensor, q_out: torch.Tensor,
+                    k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, *, num_heads: int, num_kv_heads: int,
+                    head_dim: int, value_dim: int, rotary_dim: int, page_size: int, unit_norm: bool, eps: float,
+                    store: bool = True) -> None:
+    """Rotation of the first ``rotary_dim`` dims of every q and k head, then (``unit_norm``) each
+    head divided by its root mean square over ``head_dim`` (times a weight, if given); q written to
+    q_out, k and v into pages.  Values are ``value_dim`` wide.  ``rotary_dim`` 0: no rotation."""
+    _gpu(qkv, q_weight, k_weight, cos, sin, positions, req_of_token, block_tables, q_out, k_cache, v_cache)
+    n = positions.numel()
+    nkv_in = num_kv_heads if store else 0
+    width = (num_heads + nkv_in) * head_dim + nkv_in * value_dim
+    in_f32, parts, stride = _partials(qkv, n, width, q_out.dtype, "qkv")
+    _need(q_out.numel() >= n * num_heads * head_dim, "q_out too small")
+    _need(head_dim % 8 == 0 and value_dim % 16 == 0 and max(head_dim, value_dim) <= 512 and page_size % 8 == 0,
+          "head_dim must be a multiple of 8, value_dim of 16 (at most 512), page_size of 8")
+    _need(rotary_dim % 2 == 0 and rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
+    _need(rotary_dim == 0 or (cos is not None and sin is not None and cos.dtype == torch.float32
+                               and sin.dtype == torch.float32 and cos.numel() >= n * (rotary_dim // 2)
+                               and sin.numel() >= n * (rotary_dim // 2)), "rotary tables missing, not float32 or too small")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.numel() == head_dim), "q/k norm weights are float32 [head_dim]")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32
+          and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    _need(req_of_token.numel() >= n, "req_of_token shorter than positions")
+    if store:
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_out.dtype
+              and v_cache.dtype == q_out.dtype, "cache dtype must match activations")
+        _need(k_cache.numel() % (num_kv_heads * head_dim * page_size) == 0
+              and v_cache.numel() % (num_kv_heads * value_dim * page_size) == 0
+              and k_cache.numel() // head_dim == v_cache.numel() // value_dim, "cache size is not whole pages")
+    _note(f"{n}x{width}", n * width * (qkv.element_size() * parts + q_out.element_size()))
+    _check(_fn("elementwise", "tk_rope_norm_store")(
+        _code(q_out.dtype), _p(qkv), in_f32, parts, stride, _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
+        _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
+        nkv_in, num_kv_heads, head_dim, value_dim, rotary_dim, page_size, block_tables.shape[1], int(bool(unit_norm)),
+        float(eps), _stream()), "rope_norm_store")
+
+
+def scale_softcap(logits: torch.Tensor, scale: float, cap: float | None) -> None:
+    """In place on float32 logits: x <- x * scale, then with a ``cap`` x <- cap * tanh(x / cap)."""
+    _gpu(logits)
+    _need(logits.dtype == torch.float32, "logits are float32")
+    _check(_fn("elementwise", "tk_scale_softcap")(_p(logits), logits.numel(), float(scale), float(cap or 0.0), _stream()),
+           "scale_softcap")
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
@@ -709,6 +773,77 @@ def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tens
         _code(dtype), *operands, _p(w0), _p(u), _p(gain), _p(state),
         _p(batch.q_start), _p(batch.state_slots), _p(out), batch.num_requests, heads, dim, float(eps), _stream()),
         "wkv_scan")
+
+
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, decay_in: torch.Tensor,
+             bias: torch.Tensor, gain: torch.Tensor, state: torch.Tensor, out: torch.Tensor, batch, *, heads: int,
+             dim: int, vdim: int, q_scale: float, tau: float, eps: float) -> None:
+    """Per request and head, over the step's tokens in order: S <- diag(a) S + k v^T with
+    a = sigmoid(decay_in + bias)^(1 / tau), then o = S^T (q * q_scale) (S float32 [slots, heads, dim, vdim],
+    kept); out = o / rms(o) * gain * silu(gate).  q, k, decay_in: [N, heads * dim]; v, gate: [N, heads * vdim];
+    each in out's dtype or float32, or float32 partial sums [P, N, width] of a split product."""
+    _gpu(q, k, v, gate, decay_in, bias, gain, state, out)
+    n = out.shape[0]
+    dtype = out.dtype
+    _need(out.shape[1] == heads * vdim and 1 <= dim <= WKV_MAX_DIM and 1 <= vdim <= WKV_MAX_DIM,
+          f"the scan takes heads of up to {WKV_MAX_DIM} channels")
+    _need(bias.dtype == torch.float32 and bias.numel() == heads * dim, "the decay's bias is float32 [heads * dim]")
+    _need(gain.dtype == torch.float32 and gain.numel() == vdim, "the gain is float32 [vdim]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, vdim), "the state is float32 [slots, heads, dim, vdim]")
+    _need(batch.num_tokens == n and tau > 0, "the step's descriptor does not match")
+    operands = [x for t, what, w in ((q, "q", heads * dim), (k, "k", heads * dim), (v, "v", heads * vdim),
+                                     (gate, "gate", heads * vdim), (decay_in, "decay_in", heads * dim))
+                for x in _branch(t, n, w, dtype, what)]
+    _note(f"{n}x{heads}x{dim}x{vdim}", n * heads * (3 * dim + 3 * vdim) * out.element_size(), 4.0 * n * heads * dim * vdim)
+    _check(_fn("recurrent", "tk_gla_scan")(
+        _code(dtype), *operands, _p(bias), _p(gain), _p(state), _p(batch.q_start), _p(batch.state_slots), _p(out),
+        batch.num_requests, heads, dim, vdim, float(q_scale), 1.0 / float(tau), float(eps), _stream()), "gla_scan")
+
+
+MOE_LDS_BYTES = 96 * 1024      # of a row of activations in float32 that a block of the expert kernels stages
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, top: int) -> None:
+    """Per token the ``top`` experts with the largest sigmoid(router . h), float32 throughout:
+    chosen [N, top] int32 (largest first, the lower index on ties), weight [N, top] float32 their scores."""
+    _gpu(h, router, chosen, weight)
+    n, w = h.shape
+    e = router.shape[0]
+    _need(router.dtype == torch.float32 and router.shape == (e, w), "the router is float32 [experts, width]")
+    _need(1 <= top <= e and chosen.dtype == torch.int32 and weight.dtype == torch.float32
+          and chosen.numel() >= n * top and weight.numel() >= n * top, "lists of chosen experts too small")
+    _check(_fn("moe", "tk_moe_route")(_code(h.dtype), _p(h), _p(router), _p(chosen), _p(weight), n, w, e, top, _stream()),
+           "moe_route")
+
+
+def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, act: torch.Tensor,
+                top: int) -> None:
+    """act[n * top + k] = silu(w gate_e h[n]) * (w up_e h[n]) for the token's k-th chosen expert e with
+    weight w; gate_up [experts, 2 ff, width] holds an expert's gate rows, then its up rows."""
+    _gpu(h, gate_up, chosen, weight, act)
+    n, w = h.shape
+    e, two_f, w2 = gate_up.shape
+    f = two_f // 2
+    _need(w2 == w and two_f % 2 == 0 and gate_up.dtype == h.dtype == act.dtype, "expert weights do not match the activations")
+    _need(act.shape == (n * top, f) and chosen.numel() >= n * top and weight.numel() >= n * top, "expert activations too small")
+    _need(w % (4 if h.dtype == torch.float32 else 8) == 0 and w * 4 <= MOE_LDS_BYTES, "width must fill 16-byte pieces and fit LDS")
+    _note(f"{n}x{top} {two_f}x{w}", min(n * top, e) * two_f * w * h.element_size(), 2.0 * n * top * two_f * w)
+    _check(_fn("moe", "tk_moe_gate_up")(_code(h.dtype), _p(h), _p(gate_up), _p(chosen), _p(weight), _p(act), n, w, f, top,
+                                        _stream()), "moe_gate_up")
+
+
+def moe_down(act: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, out: torch.Tensor, top: int) -> None:
+    """out[n] = sum over the token's chosen experts, in list order, of down_e act[n * top + k]; out float32 [N, width]."""
+    _gpu(act, down, chosen, out)
+    e, w, f = down.shape
+    n = out.shape[0]
+    _need(act.shape == (n * top, f) and act.dtype == down.dtype and out.dtype == torch.float32 and out.shape == (n, w),
+          "expert outputs do not match")
+    _need(f % (4 if act.dtype == torch.float32 else 8) == 0 and top * f * 4 <= MOE_LDS_BYTES,
+          "ff must fill 16-byte pieces and a token's expert activations fit LDS")
+    _note(f"{n}x{top} {w}x{f}", min(n * top, e) * w * f * act.element_size(), 2.0 * n * top * w * f)
+    _check(_fn("moe", "tk_moe_down")(_code(act.dtype), _p(act), _p(down), _p(chosen), _p(out), n, w, f, top, _stream()),
+           "moe_down")
 
 
 FEWROWS_MAX_ROWS = 64          # float32 products of up to this many rows stream the weights, a lane a weight row,
@@ -1041,22 +1176,30 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             req_of_token: torch.Tensor, out: torch.Tensor, *, num_heads: int,
                             num_kv_heads: int, head_dim: int, page_size: int, scale: float,
                             window: int | None = None, tiles: tuple | None = None,
-                            share_heads: bool | None = None) -> None:
+                            share_heads: bool | None = None, value_dim: int | None = None,
+                            chunk: int | None = None) -> None:
     """Causal attention of each query token over its request's pages.  ``tiles``:
     (tile_first, tile_count, num_tiles, single_tokens, num_single), the step's work lists (tiles
     of up to 16 consecutive tokens of one request, and token rows that run alone), which together
     name every token once; tokens of a tile share the keys and values they load.  Without it every
     token runs alone; the result is the same bit for bit.  ``share_heads``: whether the query heads
     of a group share a block (and the keys it loads) for the tokens that run alone; None chooses by
-    how many there are; the same bits again."""
+    how many there are; the same bits again.  ``value_dim``: size of a value head if it differs from
+    ``head_dim``.  ``chunk``: a query sees only the keys of its own chunk of that many positions
+    (counted from position 0); not together with ``window``."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out)
     n = positions.numel()
+    vd = head_dim if value_dim is None else int(value_dim)
+    _need(not (window and chunk), "a window or chunks, not both")
+    span = int(window or 0) if not chunk else -int(chunk)
     _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "attention tensors must share a dtype")
-    _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * head_dim, "q/out too small")
-    _need(head_dim % 16 == 0 and head_dim <= 512 and page_size % 8 == 0, "head_dim must be a multiple of 16 (at most 512), page_size a multiple of 8")
+    _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * vd, "q/out too small")
+    _need(head_dim % 8 == 0 and vd % 16 == 0 and max(head_dim, vd) <= 512 and page_size % 8 == 0,
+          "head_dim must be a multiple of 8, the value size of 16 (at most 512), page_size a multiple of 8")
     _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
     page_elems = num_kv_heads * head_dim * page_size
-    _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
+    _need(k_cache.numel() % page_elems == 0 and v_cache.numel() * head_dim == k_cache.numel() * vd,
+          "cache size is not whole pages")
     _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32
           and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
     tile_first = tile_count = single = None
@@ -1070,8 +1213,8 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                                   and single.numel() >= num_single), "bad list of single tokens")
     _check(_fn("attention_generic", "tk_paged_attention_generic")(
         _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
-        _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, page_size,
-        block_tables.shape[1], float(scale), int(window or 0), _p(tile_first), _p(tile_count), num_tiles,
+        _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, vd, page_size,
+        block_tables.shape[1], float(scale), span, _p(tile_first), _p(tile_count), num_tiles,
         _p(single), num_single, -1 if share_heads is None else int(share_heads), _stream()), "paged_attention_generic")
 
 

@@ -1,7 +1,7 @@
 """Parts a layer is made of.  Importing this package registers the built-in ones."""
 
-from tokamak_amd.parts import (attention, block, embedding, feed_forward, norm, pooled_attention,  # noqa: F401
-                               rotary, scale, time_mix)
+from tokamak_amd.parts import (attention, block, embedding, feed_forward, linear_attention, norm,  # noqa: F401
+                               pooled_attention, rotary, routed_experts, scale, time_mix)
 from tokamak_amd.parts.base import (
     Block,
     CacheRequest,

@@ -116,4 +116,89 @@ class GQAAttention(Mixer):
         return linear(attended, self.o, allow_partials=True, add_into=add_into)
 
 
+class RotatedUnitAttention(Mixer):
+    """Grouped-query attention whose queries and keys are rotated first and then each divided
+    by its root mean square per head (a unit norm without a weight), with values of a size of
+    their own and an optional chunked mask.
+
+    q = W_q h, k = W_k h (``num_heads`` / ``num_kv_heads`` heads of ``head_dim``), v = W_v h
+    (``num_kv_heads`` heads of ``value_dim``), no biases; the layer's position encoding rotates
+    the first ``rotary_dim`` dims of q and k (half-split pairs), the rest pass; then
+    q, k <- x / sqrt(mean(x^2) + ``norm_eps``) per head (``norm_eps`` None: no norm);
+    score = q . k * ``softmax_scale``; with ``chunk`` = C position i sees j <= i only if
+    i // C == j // C, chunks counted from position 0 of the sequence whatever the step's cut;
+    ordinary softmax; o projection over the concatenated heads.  Keys are cached after rotation
+    and norm, values as projected.  Tensors: q, k, v, o behind the part's prefix.
+    """
+
+    capturable = True
+    replayable = True
+
+    def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                 softmax_scale: float, norm_eps: float | None, chunk: int | None, dtype, device,
+                 names: tuple[str, str, str, str] = ("q", "k", "v", "o")) -> None:
+        super().__init__(dtype=dtype, device=device)
+        if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
+            raise ValueError(f"num_heads ({num_heads}) must be a multiple of num_kv_heads ({num_kv_heads})")
+        if head_dim % 8 or value_dim % 16 or max(head_dim, value_dim) > 512:
+            raise ValueError(f"head_dim must be a multiple of 8 and value_dim of 16, at most 512; got {head_dim}, {value_dim}")
+        if chunk is not None and chunk < 1:
+            raise ValueError(f"chunk must be >= 1, got {chunk}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.value_dim = int(head_dim), int(value_dim)
+        self.softmax_scale = float(softmax_scale)
+        self.norm_eps = None if norm_eps is None else float(norm_eps)
+        self.chunk = None if chunk is None else int(chunk)
+        self.names = tuple(names)
+        self.qkv: torch.Tensor | None = None
+        self.o: torch.Tensor | None = None
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        h, nh, nkv, hd, vd = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        q, k, v, o = self.names
+        return {prefix + q: TensorSpec((nh * hd, h)), prefix + k: TensorSpec((nkv * hd, h)),
+                prefix + v: TensorSpec((nkv * vd, h)), prefix + o: TensorSpec((h, nh * vd))}
+
+    def bind(self, prefix: str, fetch: Fetch) -> None:
+        q, k, v, o = self.names
+        self.qkv = torch.cat([fetch(prefix + n) for n in (q, k, v)], dim=0).contiguous()
+        self.o = fetch(prefix + o)
+
+    def cache_request(self) -> CacheRequest:
+        return CacheRequest.of(window=None, k=self.num_kv_heads * self.head_dim, v=self.num_kv_heads * self.value_dim)
+
+    def step_planner(self):
+        return ATTENTION_WORK
+
+    def check_page_size(self, page_size: int) -> None:
+        check_page_size(page_size)
+
+    def pair_flops(self) -> float:
+        return 2.0 * self.num_heads * (self.head_dim + self.value_dim)
+
+    def forward(self, h, batch, store, writes_cache: bool = True, position: PositionData | None = None):
+        nh, nkv, hd, vd = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        n = h.shape[0]
+        weight = self.qkv if writes_cache else self.qkv[: nh * hd]
+        qkv = linear(h, weight, allow_partials=True)
+        cos = sin = None
+        rotary_dim = 0
+        if position is not None:
+            if position.score_slopes is not None:
+                raise ops.KernelError("this attention part has no kernel for a bias on the scores")
+            cos, sin, rotary_dim = position.cos, position.sin, position.rotary_dim
+        tables = batch.block_tables[store.group]
+        q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
+        ops.rope_norm_store(
+            qkv, None, None, cos, sin, batch.positions, batch.req_of_token, tables, q, store.arrays["k"],
+            store.arrays["v"], num_heads=nh, num_kv_heads=nkv, head_dim=hd, value_dim=vd, rotary_dim=rotary_dim,
+            page_size=store.page_size, unit_norm=self.norm_eps is not None, eps=self.norm_eps or 0.0, store=writes_cache)
+        attended = torch.empty((n, nh * vd), dtype=h.dtype, device=h.device)
+        paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended, num_heads=nh,
+                        num_kv_heads=nkv, head_dim=hd, value_dim=vd, page_size=store.page_size,
+                        scale=self.softmax_scale, chunk=self.chunk)
+        return linear(attended, self.o, allow_partials=True)
+
+
 register_part("mixer", "gqa_attention", GQAAttention)
+register_part("mixer", "rotated_unit_attention", RotatedUnitAttention)

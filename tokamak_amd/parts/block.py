@@ -18,25 +18,30 @@ class PreNormBlock(Block):
     (``fuses_residual``) are offered the stream itself, so that in a decode step
     of few rows their last product adds into it and the next product finishes
     the norm, with no kernel in between.  An optional ``position`` part prepares
-    the step's position data for the mixer.
+    the step's position data for the mixer.  The feed-forward and its norm may be
+    absent together: the layer is then x = x + mixer(norm(x)) alone.
     """
 
-    roles = ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")
-    optional = ("position",)
+    roles = ("mixer_norm", "mixer")
+    optional = ("position", "feed_forward_norm", "feed_forward")
     fuses_residual = True
     replays_parts = True
 
     def __init__(self, parts) -> None:
         super().__init__(parts)
         self.mixer_norm = parts["mixer_norm"]
-        self.feed_forward_norm = parts["feed_forward_norm"]
-        self.feed_forward = parts["feed_forward"]
+        self.feed_forward_norm = parts.get("feed_forward_norm")
+        self.feed_forward = parts.get("feed_forward")
+        if (self.feed_forward is None) != (self.feed_forward_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.position = parts.get("position")
         self.entry_norm = self.mixer_norm
 
     def forward(self, resid, pending, batch, store, writes_cache, then=None):
         position = None if self.position is None else self.position.prepare(batch)
         h = _normed(self.mixer_norm, resid, pending, self.mixer)
+        if self.feed_forward is None:
+            return self.mixer.forward(h, batch, store, writes_cache, position, **_sink(self.mixer, then, resid))
         into = _sink(self.mixer, self.feed_forward_norm, resid)
         pending = self.mixer.forward(h, batch, store, writes_cache, position, **into)
         h = _normed(self.feed_forward_norm, resid, pending, self.feed_forward)

@@ -12,14 +12,16 @@ from tokamak_amd.weights.spec import TensorSpec
 
 
 class TokenEmbedding(Embedding):
-    """Plain row gather into the float32 residual stream, no scaling
-    (reference: src/tokamak/model/transformer.py:140)."""
+    """Row gather into the float32 residual stream (reference: src/tokamak/model/transformer.py:140),
+    times ``scale`` if the design has one.  ``add_to`` adds the same rows into a stream once more,
+    for a model that feeds its input in again further up (``LayerCall.adds_embedding``)."""
 
     capturable = True
 
-    def __init__(self, *, vocab_size: int, dim: int, dtype, device, tensor: str = "weight") -> None:
+    def __init__(self, *, vocab_size: int, dim: int, dtype, device, tensor: str = "weight", scale: float = 1.0) -> None:
         super().__init__(dtype=dtype, device=device)
         self.vocab_size, self.dim = int(vocab_size), int(dim)
+        self.scale = float(scale)
         self.tensor = str(tensor)       # the matrix's name behind the part's prefix
         self.weight: torch.Tensor | None = None
 
@@ -34,19 +36,28 @@ class TokenEmbedding(Embedding):
 
     def forward(self, batch) -> torch.Tensor:
         resid = torch.empty((batch.num_tokens, self.dim), dtype=torch.float32, device=self.device)
-        ops.embed_gather(self.weight, batch.token_ids, resid)
+        ops.embed_gather(self.weight, batch.token_ids, resid, self.scale)
         return resid
+
+    def add_to(self, batch, resid: torch.Tensor) -> None:
+        ops.embed_gather(self.weight, batch.token_ids, resid, self.scale, accumulate=True)
 
 
 class LinearHead(Head):
     """logits = h @ W^T in float32; a tied head uses the embedding matrix itself
-    (reference: src/tokamak/model/transformer.py:154-156,173-176)."""
+    (reference: src/tokamak/model/transformer.py:154-156,173-176).  With ``scale`` the logits
+    are multiplied by it, and with ``softcap`` c they then become c * tanh(logits / c)."""
 
     capturable = True
 
-    def __init__(self, *, vocab_size: int, dim: int, tied: bool, dtype, device, tensor: str = "weight") -> None:
+    def __init__(self, *, vocab_size: int, dim: int, tied: bool, dtype, device, tensor: str = "weight",
+                 scale: float = 1.0, softcap: float | None = None) -> None:
         super().__init__(dtype=dtype, device=device)
         self.vocab_size, self.dim, self.tied = int(vocab_size), int(dim), bool(tied)
+        self.scale = float(scale)
+        self.softcap = None if softcap is None else float(softcap)
+        if self.softcap is not None and self.softcap <= 0:
+            raise ValueError(f"softcap must be positive, got {softcap}")
         self.tensor = str(tensor)
         self.weight: torch.Tensor | None = None
 
@@ -67,7 +78,10 @@ class LinearHead(Head):
         self.weight = weight
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return linear(h, self.weight, out_dtype=torch.float32)
+        logits = linear(h, self.weight, out_dtype=torch.float32)
+        if self.scale != 1.0 or self.softcap is not None:
+            ops.scale_softcap(logits, self.scale, self.softcap)
+        return logits
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

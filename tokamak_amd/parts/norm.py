@@ -17,16 +17,19 @@ class RMSNorm(Norm):
     Statistics and the product with the weight are float32; one rounding to the
     compute dtype at the end (reference: src/tokamak/model/layers.py:28-33
     computes the statistics in float32, rounds, then multiplies by the weight).
+    ``offset``: the checkpoint stores the weight less this number (a weight kept around
+    zero has offset 1); it is added once, in float32, at binding.
     """
 
     capturable = True
     fuses_residual = True
     replayable = True
 
-    def __init__(self, *, dim: int, eps: float, dtype, device, tensor: str = "weight") -> None:
+    def __init__(self, *, dim: int, eps: float, dtype, device, tensor: str = "weight", offset: float = 0.0) -> None:
         super().__init__(dtype=dtype, device=device)
         self.dim = int(dim)
         self.eps = float(eps)
+        self.offset = float(offset)
         self.tensor = str(tensor)       # the weight's name behind the part's prefix
         self.weight: torch.Tensor | None = None
 
@@ -35,6 +38,8 @@ class RMSNorm(Norm):
 
     def bind(self, prefix: str, fetch: Fetch) -> None:
         self.weight = fetch(prefix + self.tensor)
+        if self.offset != 0.0:
+            self.weight = (self.weight + self.offset).contiguous()
 
     def sink(self, resid: torch.Tensor) -> StreamSink:
         return StreamSink(resid, self.weight)

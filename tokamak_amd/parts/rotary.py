@@ -17,20 +17,29 @@ class RotaryHalf(PositionEncoding):
     float(pos) * inv_freq[j] and its cos/sin are float32 (layers.py:56-58).  The
     rotation itself pairs dim j with dim j + rotary_dim/2 (layers.py:61-63) and
     is applied by the mixer's fused kernel.
+
+    ``scaling`` = (factor, low, high, original) rescales the frequencies by wavelength
+    l = 2 pi / f: kept where l < original / high, divided by ``factor`` where l > original / low,
+    and in between (1 - s) f / factor + s f with s = (original / l - low) / (high - low);
+    computed on the host in double precision, then rounded to float32 once.
     """
 
     capturable = True
     replayable = True
 
-    def __init__(self, *, rotary_dim: int, theta: float, dtype, device) -> None:
+    def __init__(self, *, rotary_dim: int, theta: float, dtype, device, scaling: tuple | None = None) -> None:
         super().__init__(dtype=dtype, device=device)
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim must be even, got {rotary_dim}")
         self.rotary_dim = int(rotary_dim)
         self.theta = float(theta)
-        inv_freq = 1.0 / (self.theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+        self.scaling = None if scaling is None else tuple(float(x) for x in scaling)
+        if self.scaling is None:
+            inv_freq = 1.0 / (self.theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+        else:
+            inv_freq = torch.tensor(scaled_frequencies(self.rotary_dim, self.theta, *self.scaling), dtype=torch.float32)
         self.inv_freq = inv_freq.to(self.device)
-        self.key = ("rotary_half", self.rotary_dim, self.theta)
+        self.key = ("rotary_half", self.rotary_dim, self.theta, self.scaling)
 
     def prepare(self, batch) -> PositionData:
         """cos and sin, each float32 [N, rotary_dim/2]; computed once per step."""
@@ -42,6 +51,27 @@ class RotaryHalf(PositionEncoding):
             ops.rope_tables(batch.positions, self.inv_freq, cos, sin)
             cached = batch.memo[self.key] = PositionData(cos=cos, sin=sin, rotary_dim=self.rotary_dim)
         return cached
+
+
+def scaled_frequencies(rotary_dim: int, theta: float, factor: float, low: float, high: float, original: float) -> list[float]:
+    """theta^(-2j / rotary_dim) for j < rotary_dim / 2, rescaled by wavelength (see ``RotaryHalf``)."""
+    import math
+
+    if factor <= 0 or high <= low or original <= 0:
+        raise ValueError("frequency scaling needs factor > 0, high > low and original > 0")
+    out = []
+    for j in range(rotary_dim // 2):
+        f = theta ** (-2.0 * j / rotary_dim)
+        turns = original * f / (2.0 * math.pi)      # original / wavelength
+        if turns > high:
+            pass
+        elif turns < low:
+            f /= factor
+        else:
+            s = (turns - low) / (high - low)
+            f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return out
 
 
 register_part("position", "rotary_half", RotaryHalf)

@@ -1,0 +1,71 @@
+"""A routed feed-forward: a mixture of small gated experts."""
+
+from __future__ import annotations
+
+import torch
+
+from tokamak_amd.config.registry import register_part
+from tokamak_amd.kernels import ops
+from tokamak_amd.parts.base import FeedForward, Fetch
+from tokamak_amd.weights.spec import TensorSpec
+
+
+class RoutedExperts(FeedForward):
+    """``num_experts`` feed-forwards down(silu(gate x) * up x) without biases, of which every token
+    uses ``top``.
+
+    The router's logits z = W_r h and the scores s = sigmoid(z) are float32; the ``top`` experts
+    with the largest scores are chosen (the lower index on a tie) and weighted by their scores
+    as they are, not renormalised.  ``weight_on`` says where a weight w acts: ``"input"``, the
+    expert sees w * h (out = sum expert(w h)), or ``"output"``, out = sum w * expert(h).  On the
+    input the kernels use gate(w h) = w gate(h): the weight scales the two first products in
+    float32.  Tensors: router, e<i>.gate, e<i>.up, e<i>.down; an expert's gate and up are held as
+    one matrix and the experts as one array each.
+    """
+
+    capturable = True
+    replayable = True
+
+    def __init__(self, *, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
+                 weight_on: str = "input", dtype, device,
+                 names: tuple[str, str, str, str, str] = ("router", "e{}.", "gate", "up", "down")) -> None:
+        super().__init__(dtype=dtype, device=device)
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.num_experts, self.top = int(num_experts), int(top)
+        if not 1 <= self.top <= self.num_experts:
+            raise ValueError(f"top ({top}) must be between 1 and the number of experts ({num_experts})")
+        if weight_on != "input":
+            raise ValueError(f"the expert kernels weigh an expert's input; weight_on={weight_on!r} has no kernel")
+        self.weight_on = weight_on
+        self.names = tuple(names)
+        self.router = self.gate_up = self.down = None
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        h, f = self.hidden_size, self.intermediate_size
+        router, expert, gate, up, down = self.names
+        out = {prefix + router: TensorSpec((self.num_experts, h), held="float32")}
+        for e in range(self.num_experts):
+            base = prefix + expert.format(e)
+            out.update({base + gate: TensorSpec((f, h)), base + up: TensorSpec((f, h)), base + down: TensorSpec((h, f))})
+        return out
+
+    def bind(self, prefix: str, fetch: Fetch) -> None:
+        router, expert, gate, up, down = self.names
+        self.router = fetch(prefix + router)
+        bases = [prefix + expert.format(e) for e in range(self.num_experts)]
+        self.gate_up = torch.stack([torch.cat([fetch(b + gate), fetch(b + up)], dim=0) for b in bases]).contiguous()
+        self.down = torch.stack([fetch(b + down) for b in bases]).contiguous()
+
+    def forward(self, h, batch):
+        n, top = h.shape[0], self.top
+        chosen = torch.empty((n, top), dtype=torch.int32, device=h.device)
+        weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
+        ops.moe_route(h, self.router, chosen, weight, top)
+        act = torch.empty((n * top, self.intermediate_size), dtype=h.dtype, device=h.device)
+        ops.moe_gate_up(h, self.gate_up, chosen, weight, act, top)
+        out = torch.empty((n, self.hidden_size), dtype=torch.float32, device=h.device)
+        ops.moe_down(act, self.down, chosen, out, top)
+        return out
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)
