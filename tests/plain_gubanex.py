@@ -77,16 +77,15 @@ def chunked_attention(h: torch.Tensor, w: dict, prefix: str, m: dict, eps: float
     q, k = rms(rotate(q, positions, freqs), eps), rms(rotate(k, positions, freqs), eps)
     if past is not None:
         k, v = torch.cat([past[0], k]), torch.cat([past[1], v])
-    size = int(m["mask"]["size"])
+    size = int(m["mask"]["size"]) if m.get("mask") else None
+    group = heads // kv
     out = torch.zeros(t, heads, vdim, dtype=h.dtype)
     for a in range(t):
         i = first_position + a
-        seen = [j for j in range(i + 1) if chunk_visible(i, j, size)]
+        seen = [j for j in range(i + 1) if size is None or chunk_visible(i, j, size)]
         for head in range(heads):
-            g = head // (heads // kv)
-            scores = torch.stack([(q[a, head] * k[j, g]).sum() for j in seen]) * float(m["scale"])
-            p = torch.softmax(scores, dim=0)
-            out[a, head] = (p[:, None] * v[seen, g]).sum(0)
+            scores = (k[seen, head // group] @ q[a, head]) * float(m["scale"])
+            out[a, head] = torch.softmax(scores, dim=0) @ v[seen, head // group]
     return out.reshape(t, heads * vdim) @ w[prefix + "o"].T, (k, v)
 
 
@@ -109,13 +108,20 @@ def gated_linear_attention(h: torch.Tensor, w: dict, prefix: str, m: dict, eps: 
     return out.reshape(t, heads * vdim) @ w[prefix + "o"].T, s
 
 
-def routed_experts(h: torch.Tensor, w: dict, prefix: str, mlp: dict) -> torch.Tensor:
-    """Sigmoid router; the chosen experts' scores weigh the experts' INPUT and are not renormalised."""
+def routed_experts(h: torch.Tensor, w: dict, prefix: str, mlp: dict, margins: list | None = None) -> torch.Tensor:
+    """Sigmoid router; the chosen experts' scores weigh the experts' INPUT and are not renormalised.
+    ``margins`` receives, per token, how far the last chosen expert's logit lies above the first one
+    left out, relative to their size (infinite if every expert is chosen)."""
     experts, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
-    scores = torch.sigmoid(h @ w[prefix + "router"].T)
+    z = h @ w[prefix + "router"].T
+    scores = torch.sigmoid(z)
     out = torch.zeros_like(h)
     for a in range(h.shape[0]):
-        chosen = sorted(range(experts), key=lambda e: (-float(scores[a, e]), e))[:top]
+        order = sorted(range(experts), key=lambda e: (-float(scores[a, e]), e))
+        chosen = order[:top]
+        if margins is not None:
+            last, nxt = (float(z[a, order[top - 1]]), float(z[a, order[top]])) if top < experts else (math.inf, 0.0)
+            margins.append((last - nxt) / (abs(last) + abs(nxt) + 1.0) if top < experts else math.inf)
         for e in chosen:
             x = scores[a, e] * h[a]
             name = f"{prefix}e{e}."
@@ -147,14 +153,16 @@ class PlainGubanex:
         self.calls = layer_calls(cfg)
         self.kept: list = [None] * len(self.calls)
         self.length = 0
+        self.margins: list[float] = []      # per position, the narrowest choice of experts in any layer call
 
     def forward(self, tokens: list[int], trace: list | None = None) -> torch.Tensor:
         """Logits [T, vocab] for the next ``tokens`` of the sequence.  ``trace`` receives the stream
         after every layer call."""
         cfg, w = self.cfg, self.w
         eps = float(cfg["norm"]["eps"])
-        embedded = w["embed"][torch.tensor(tokens)] * float(cfg["embedding"]["scale"])
+        embedded = w["embed"][torch.tensor(tokens)] * float(cfg.get("embedding", {}).get("scale", 1.0))
         x = embedded.clone()
+        narrowest = [math.inf] * len(tokens)
         for at, (i, add) in enumerate(self.calls):
             layer, base = cfg["layers"][i], f"l{i}."
             if add:
@@ -168,10 +176,15 @@ class PlainGubanex:
                 raise ValueError(layer["type"])
             x = x + y
             if layer.get("mlp") is not None:
-                x = x + routed_experts(offset_norm(x, w[base + "norm2"], eps), w, base + "mlp.", layer["mlp"])
+                margins: list[float] = []
+                x = x + routed_experts(offset_norm(x, w[base + "norm2"], eps), w, base + "mlp.", layer["mlp"], margins)
+                narrowest = [min(a, b) for a, b in zip(narrowest, margins)]
             if trace is not None:
                 trace.append(x.clone())
         self.length += len(tokens)
-        logits = (offset_norm(x, w["final.norm"], eps) @ w["head"].T) * float(cfg["logit_scale"])
+        self.margins += narrowest
+        logits = (offset_norm(x, w["final.norm"], eps) @ w["head"].T) * float(cfg.get("logit_scale", 1.0))
+        if cfg.get("logit_softcap") is None:
+            return logits
         cap = float(cfg["logit_softcap"])
         return cap * torch.tanh(logits / cap)

@@ -195,11 +195,17 @@ def test_a_block_says_which_parts_it_needs():
 
     plan = qwen3.plan(qwen3.parse(raw(), ()))
     layer = plan.layers[0]
-    broken = LayerSpec(tuple((r, p) for r, p in layer.parts if r != "feed_forward_norm")
+    broken = LayerSpec(tuple((r, p) for r, p in layer.parts if r != "mixer_norm")
                        + (("extra", SubPart("norm", layer.role("mixer_norm").spec, "x.")),), layer.block)
     import dataclasses
-    with pytest.raises(ValueError, match="missing \\['feed_forward_norm'\\], unknown \\['extra'\\]"):
+    with pytest.raises(ValueError, match="missing \\['mixer_norm'\\], unknown \\['extra'\\]"):
         LayeredModel(dataclasses.replace(plan, layers=(broken, broken)), dtype=torch.float32, device="meta")
+    # the feed-forward and its norm may be absent, but only together
+    halved = LayerSpec(tuple((r, p) for r, p in layer.parts if r != "feed_forward_norm"), layer.block)
+    with pytest.raises(ValueError, match="come together"):
+        LayeredModel(dataclasses.replace(plan, layers=(halved, halved)), dtype=torch.float32, device="meta")
+    bare = LayerSpec(tuple((r, p) for r, p in layer.parts if not r.startswith("feed_forward")), layer.block)
+    assert LayeredModel(dataclasses.replace(plan, layers=(bare, bare)), dtype=torch.float32, device="meta").blocks[0].feed_forward is None
     model = LayeredModel(plan, dtype=torch.float32, device="meta")
     assert model.blocks[0].parts["position"] is model.blocks[1].parts["position"]      # shared: one table a step
     assert model.blocks[0].parts["mixer"] is not model.blocks[1].parts["mixer"]

@@ -87,7 +87,14 @@ __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
 
 // a[p, c] = silu(w g) * (w u), g = Wg[e][c] . h[n], u = Wu[e][c] . h[n]; gate_up [E][2 F][W]
 // (an expert's gate rows, then its up rows).  grid (pairs, slabs of channels).
-template <typename T>
+// WIDE: rows are walked in 16-byte pieces (their length fills such pieces), else element by element.
+template <typename T, bool WIDE>
+__device__ __forceinline__ void load_piece(const T* p, float* o) {
+  if constexpr (WIDE) Vec<T>::load(p, o);
+  else o[0] = Elem<T>::load(p);
+}
+
+template <typename T, bool WIDE>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(
     const T* __restrict__ h, const T* __restrict__ gate_up, const int* __restrict__ chosen,
     const float* __restrict__ weight, T* __restrict__ act, int W, int F, int top, int slab) {
@@ -100,7 +107,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
   const float wt = weight[p];
   const T* wg = gate_up + (size_t)e * 2 * F * W;
   const T* wu = wg + (size_t)F * W;
-  constexpr int V = Vec<T>::N;
+  constexpr int V = WIDE ? Vec<T>::N : 1;
   const int c_end = min(F, (int)(blockIdx.y + 1) * slab);
   for (int c0 = blockIdx.y * slab + wave * kRows; c0 < c_end; c0 += nwaves * kRows) {
     float g[kRows], u[kRows];
@@ -114,8 +121,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
       for (int r = 0; r < kRows; ++r) {
         const int c = min(c0 + r, F - 1);       // (a row past the end is walked again and not used)
         float a[V], b[V];
-        Vec<T>::load(wg + (size_t)c * W + d, a);
-        Vec<T>::load(wu + (size_t)c * W + d, b);
+        load_piece<T, WIDE>(wg + (size_t)c * W + d, a);
+        load_piece<T, WIDE>(wu + (size_t)c * W + d, b);
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           g[r] = fmaf(a[i], xv[i], g[r]);
@@ -142,7 +149,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
 
 // out[n, c] = sum over the token's chosen experts, in list order, of Wd[e][c] . a[p]; down [E][W][F];
 // out float32.  grid (tokens, slabs of columns).
-template <typename T>
+template <typename T, bool WIDE>
 __global__ __launch_bounds__(256) void moe_down_kernel(
     const T* __restrict__ act, const T* __restrict__ down, const int* __restrict__ chosen,
     float* __restrict__ out, int W, int F, int top, int slab) {
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
   for (int d = threadIdx.x; d < top * F; d += blockDim.x) x[d] = Elem<T>::load(act + (size_t)n * top * F + d);
   __syncthreads();
-  constexpr int V = Vec<T>::N;
+  constexpr int V = WIDE ? Vec<T>::N : 1;
   const int c_end = min(W, (int)(blockIdx.y + 1) * slab);
   for (int c0 = blockIdx.y * slab + wave * kRows; c0 < c_end; c0 += nwaves * kRows) {
     float total[kRows];
@@ -171,7 +178,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
         for (int r = 0; r < kRows; ++r) {
           const int c = min(c0 + r, W - 1);
           float a[V];
-          Vec<T>::load(wd + (size_t)c * F + d, a);
+          load_piece<T, WIDE>(wd + (size_t)c * F + d, a);
 #pragma unroll
           for (int i = 0; i < V; ++i) acc[r] = fmaf(a[i], xv[i], acc[r]);
         }
@@ -217,25 +224,27 @@ static int slab_for(int channels, long rows) {
 TK_API int tk_moe_gate_up(int dtype, const void* h, const void* gate_up, const int* chosen, const float* weight,
                           void* act, int N, int W, int F, int top, hipStream_t stream) {
   if (N <= 0) return 0;
-  const int vec = dtype == 0 ? 4 : 8;
-  if (W % vec != 0 || (size_t)W * 4 > 96 * 1024 || (long)N * top > 0x7fffffffL / 2) return -1;
+  const bool wide = W % (dtype == 0 ? 4 : 8) == 0;
+  if ((size_t)W * 4 > 96 * 1024 || (long)N * top > 0x7fffffffL / 2) return -1;
   const int slab = slab_for(F, (long)N * top);
   const dim3 grid(N * top, (F + slab - 1) / slab);
   const size_t lds = (size_t)W * sizeof(float);
-#define TK_GU(T_)                                                                                      \
+#define TK_GU(T_, WIDE_)                                                                               \
   {                                                                                                    \
     static bool allowed = false;                                                                       \
     if (!allowed) {                                                                                    \
-      const hipError_t err = hipFuncSetAttribute((const void*)moe_gate_up_kernel<T_>,                  \
+      const hipError_t err = hipFuncSetAttribute((const void*)moe_gate_up_kernel<T_, WIDE_>,           \
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); \
       if (err != hipSuccess) return (int)err;                                                          \
       allowed = true;                                                                                  \
     }                                                                                                  \
-    moe_gate_up_kernel<T_><<<grid, 256, lds, stream>>>((const T_*)h, (const T_*)gate_up, chosen, weight, \
-                                                       (T_*)act, W, F, top, slab);                     \
+    moe_gate_up_kernel<T_, WIDE_><<<grid, 256, lds, stream>>>((const T_*)h, (const T_*)gate_up, chosen, weight, \
+                                                              (T_*)act, W, F, top, slab);              \
   }
-  if (dtype == 0) TK_GU(float)
-  else TK_GU(bf16_t)
+  if (dtype == 0 && wide) TK_GU(float, true)
+  else if (dtype == 0) TK_GU(float, false)
+  else if (wide) TK_GU(bf16_t, true)
+  else TK_GU(bf16_t, false)
 #undef TK_GU
   return launch_status();
 }
@@ -244,24 +253,26 @@ TK_API int tk_moe_gate_up(int dtype, const void* h, const void* gate_up, const i
 TK_API int tk_moe_down(int dtype, const void* act, const void* down, const int* chosen, float* out, int N, int W,
                        int F, int top, hipStream_t stream) {
   if (N <= 0) return 0;
-  const int vec = dtype == 0 ? 4 : 8;
-  if (F % vec != 0 || (size_t)top * F * 4 > 96 * 1024) return -1;
+  const bool wide = F % (dtype == 0 ? 4 : 8) == 0;
+  if ((size_t)top * F * 4 > 96 * 1024) return -1;
   const int slab = slab_for(W, N);
   const dim3 grid(N, (W + slab - 1) / slab);
   const size_t lds = (size_t)top * F * sizeof(float);
-#define TK_DN(T_)                                                                                      \
+#define TK_DN(T_, WIDE_)                                                                               \
   {                                                                                                    \
     static bool allowed = false;                                                                       \
     if (!allowed) {                                                                                    \
-      const hipError_t err = hipFuncSetAttribute((const void*)moe_down_kernel<T_>,                     \
+      const hipError_t err = hipFuncSetAttribute((const void*)moe_down_kernel<T_, WIDE_>,              \
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); \
       if (err != hipSuccess) return (int)err;                                                          \
       allowed = true;                                                                                  \
     }                                                                                                  \
-    moe_down_kernel<T_><<<grid, 256, lds, stream>>>((const T_*)act, (const T_*)down, chosen, out, W, F, top, slab); \
+    moe_down_kernel<T_, WIDE_><<<grid, 256, lds, stream>>>((const T_*)act, (const T_*)down, chosen, out, W, F, top, slab); \
   }
-  if (dtype == 0) TK_DN(float)
-  else TK_DN(bf16_t)
+  if (dtype == 0 && wide) TK_DN(float, true)
+  else if (dtype == 0) TK_DN(float, false)
+  else if (wide) TK_DN(bf16_t, true)
+  else TK_DN(bf16_t, false)
 #undef TK_DN
   return launch_status();
 }

@@ -826,7 +826,7 @@ def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, chosen: torch.Tensor, we
     f = two_f // 2
     _need(w2 == w and two_f % 2 == 0 and gate_up.dtype == h.dtype == act.dtype, "expert weights do not match the activations")
     _need(act.shape == (n * top, f) and chosen.numel() >= n * top and weight.numel() >= n * top, "expert activations too small")
-    _need(w % (4 if h.dtype == torch.float32 else 8) == 0 and w * 4 <= MOE_LDS_BYTES, "width must fill 16-byte pieces and fit LDS")
+    _need(w * 4 <= MOE_LDS_BYTES, "a row of activations must fit LDS")
     _note(f"{n}x{top} {two_f}x{w}", min(n * top, e) * two_f * w * h.element_size(), 2.0 * n * top * two_f * w)
     _check(_fn("moe", "tk_moe_gate_up")(_code(h.dtype), _p(h), _p(gate_up), _p(chosen), _p(weight), _p(act), n, w, f, top,
                                         _stream()), "moe_gate_up")
@@ -839,8 +839,7 @@ def moe_down(act: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, out: t
     n = out.shape[0]
     _need(act.shape == (n * top, f) and act.dtype == down.dtype and out.dtype == torch.float32 and out.shape == (n, w),
           "expert outputs do not match")
-    _need(f % (4 if act.dtype == torch.float32 else 8) == 0 and top * f * 4 <= MOE_LDS_BYTES,
-          "ff must fill 16-byte pieces and a token's expert activations fit LDS")
+    _need(top * f * 4 <= MOE_LDS_BYTES, "a token's expert activations must fit LDS")
     _note(f"{n}x{top} {w}x{f}", min(n * top, e) * w * f * act.element_size(), 2.0 * n * top * w * f)
     _check(_fn("moe", "tk_moe_down")(_code(act.dtype), _p(act), _p(down), _p(chosen), _p(out), n, w, f, top, _stream()),
            "moe_down")
