@@ -137,29 +137,47 @@ class StepCost:
         tensors = {n: s for n, s in model.expected_tensors().items() if not s.ignored}
         size = {n: (4 if s.role != "matrix" else elem) for n, s in tensors.items()}
         numel = {n: _prod(s.shape) for n, s in tensors.items()}
-        embedding = set(model.embedding.expected_tensors(plan.embedding_prefix))
-        head = {n for n in model.head.expected_tensors(plan.head_prefix) if n in tensors}
         self.hidden = plan.hidden_size
         self.elem = elem
-        # every tensor a decode step reads whole: all but the embedding table (a row a token),
-        # unless the head is tied to it
-        self.weight_bytes = sum(numel[n] * size[n] for n in tensors if n not in embedding or plan.tie_word_embeddings)
         self.embedding_row_bytes = plan.hidden_size * elem
-        self.matrix_params = sum(numel[n] for n, s in tensors.items()
-                                 if s.role == "matrix" and n not in embedding and n not in head)
         self.head_params = plan.vocab_size * plan.hidden_size
+        # every tensor a decode step reads whole: all but the embedding table (a row a token),
+        # unless the head is tied to it; a part that chooses among its matrices token by token
+        # (routed experts) says which share of them a token meets and a step reads
+        self.fixed_bytes = 0.0
+        self.parts: list[tuple[object, float, float]] = []     # (part, its matrix bytes, its matrix elements)
+        for prefix, part in model._named_parts():
+            names = [n for n in part.expected_tensors(prefix) if n in tensors]
+            if part is model.embedding and not plan.tie_word_embeddings:
+                continue
+            self.fixed_bytes += sum(numel[n] * size[n] for n in names if tensors[n].role != "matrix")
+            matrices = [n for n in names if tensors[n].role == "matrix"]
+            counted = 0.0 if part in (model.embedding, model.head) else float(sum(numel[n] for n in matrices))
+            self.parts.append((part, float(sum(numel[n] * size[n] for n in matrices)), counted))
+        # a layer named several times in the run order multiplies with its matrices every time
+        calls: dict[int, int] = {}
+        for call in plan.order:
+            calls[call.layer] = calls.get(call.layer, 0) + 1
+        self.times = {id(p): calls[i] for i, block in enumerate(model.blocks) for p in block.parts.values() if i in calls}
         _, layouts = model.cache_layout()
-        self.kv_bytes_per_token = sum(lay.request.bytes_per_token(runner.dtype) for lay in layouts.values())
-        # attention flops of a layer call: 4 * heads * head_dim per (query, visible key) pair
-        self.pair_flops = sum(mixer.pair_flops() for call in plan.order
-                              for mixer in model.blocks[call.layer].mixers.values())
+        # (mixer, bytes a cached token of its slot holds, flops per visible pair) of every layer call
+        self.mixers = []
+        for call in plan.order:
+            for mixer, slot in model._mixers_of(call):
+                lay = layouts.get(slot)
+                self.mixers.append((mixer, lay.request.bytes_per_token(runner.dtype) if lay is not None else 0, mixer.pair_flops()))
 
     def decode_bytes(self, batch: int, mean_keys: float) -> float:
-        return self.weight_bytes + batch * (self.embedding_row_bytes + mean_keys * self.kv_bytes_per_token)
+        weights = self.fixed_bytes + sum(nbytes * part.matrix_share(batch)[1] for part, nbytes, _ in self.parts)
+        at = max(int(mean_keys) - 1, 0)
+        cache = sum(per_token * mixer.visible_keys(at) for mixer, per_token, _ in self.mixers)
+        return weights + batch * (self.embedding_row_bytes + cache)
 
     def prefill_flops(self, tokens: int) -> float:
-        return (2.0 * tokens * self.matrix_params + self.pair_flops * tokens * (tokens + 1) / 2
-                + 2.0 * self.head_params)
+        products = sum(2.0 * tokens * elems * part.matrix_share(tokens)[0] * self.times.get(id(part), 1)
+                       for part, _, elems in self.parts)
+        pairs = sum(flops * sum(mixer.visible_keys(p) for p in range(tokens)) for mixer, _, flops in self.mixers if flops)
+        return products + pairs + 2.0 * self.head_params
 
 
 def _prod(shape) -> int:
@@ -727,7 +745,8 @@ def main() -> int:
     ap.add_argument("--shape", default="qwen3-8b",
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
     ap.add_argument("--pairs", default="rorosun-0.6b:qwen3-0.6b,rorosun-8b:qwen3-8b",
-                    help="compare workload: NEW:OLD preset pairs, each measured like --shape")
+                    help="compare workload: NEW:OLD preset pairs, each measured like --shape "
+                         "(for instance gubanex-0.6b:qwen3-0.6b,gubanex-8b:qwen3-8b)")
     ap.add_argument("--requests", type=int, default=256)
     ap.add_argument("--max-batch", type=int, default=64)
     ap.add_argument("--prompt-tokens", default="32,1024", help="continuous workload: MIN,MAX prompt length")

@@ -228,6 +228,12 @@ def test_chunked_attention_alone(dtype, a):
     close(torch.cat(got), want, dtype)
 
 
+def clear_of(h, w, top, n):
+    """The rows whose choice of experts is no close call."""
+    scores = torch.sigmoid(h.double() @ w["l0.mlp.router"].double().T).sort(dim=1, descending=True).values
+    return torch.ones(h.shape[0], dtype=torch.bool) if top == n else (scores[:, top - 1] - scores[:, top]) > 1e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("width,ff,n,top", [(64, 32, 4, 2), (48, 24, 12, 1), (72, 40, 5, 5), (36, 20, 7, 3), (256, 136, 3, 2)])
 def test_routed_experts_alone(dtype, width, ff, n, top):
@@ -244,10 +250,12 @@ def test_routed_experts_alone(dtype, width, ff, n, top):
     g = torch.Generator().manual_seed(3)
     h = torch.randn(70, width, generator=g).to(dtype)
     want = plain.routed_experts(h.double(), double(w), "l0.mlp.", cfg["layers"][0]["mlp"]).float()
-    got = part.forward(h.to(DEV), make_batch([(70, 0, [0])])).cpu()
-    assert got.dtype == torch.float32
-    scores = torch.sigmoid(h.double() @ w["l0.mlp.router"].double().T).sort(dim=1, descending=True).values
-    clear = torch.ones(70, dtype=torch.bool) if top == n else (scores[:, top - 1] - scores[:, top]) > 1e-3
+    got = part.forward(h.to(DEV), make_batch([(70, 0, [0])]))
+    assert got.dtype == torch.float32 and got.shape == (top, 70, width)      # a layer per chosen expert, added by the reader
+    got = got.sum(0).cpu()
+    few = part.forward(h[:9].to(DEV), make_batch([(9, 0, [0])])).sum(0).cpu()   # the form for few tokens
+    close(few[clear_of(h[:9], w, top, n)], want[:9][clear_of(h[:9], w, top, n)], dtype)
+    clear = clear_of(h, w, top, n)
     assert int(clear.sum()) >= 60
     close(got[clear], want[clear], dtype)
     # the weight acts on the expert's input: it is not the same as weighting the output

@@ -8,8 +8,17 @@
 //   LDS in float32, a wave walks eight weight rows at a time in 16-byte pieces.  The weight of a
 //   chosen expert multiplies the expert's INPUT: since the first products are linear,
 //   gate(w h) = w gate(h), the weight is applied to the two products in float32 before the
-//   activation.  moe_down adds a token's experts in the order of its list, so a token's result
-//   does not depend on what else is in the step.
+//   activation.  moe_down writes every pair's result to its own row of a float32 array
+//   [top][tokens][width]; the kernel that reads it next (the norm that adds a sub-layer's output
+//   to the stream) sums the `top` layers in order, so a token's result does not depend on what
+//   else is in the step.
+// moe_sort / moe_grouped, the form for many tokens in bfloat16: the (token, expert) pairs are
+//   counted and listed expert by expert and cut into tiles of up to 64 pairs of one expert; a block
+//   takes a tile and 128 output channels on the matrix cores (v_mfma_f32_16x16x32_bf16, weights and
+//   activations as operands straight from memory), so an expert's weights are read once per 64 of
+//   its tokens.  The second product writes every pair's result to its own row of a float32 array
+//   [top][tokens][width], which the kernel that reads it next (the norm that adds a sub-layer's
+//   output to the stream) sums in list order: no block adds into another's result.
 //
 // Router, scores, weights and every sum are float32 whatever the storage type.
 #include "common.h"
@@ -54,12 +63,37 @@ __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
   if (n >= N) return;                  // nothing below synchronises across waves
   float* score = lds + (size_t)wave * E;
   const T* row = h + (size_t)n * W;
-  for (int e = 0; e < E; ++e) {
-    const float* r = router + (size_t)e * W;
-    float acc = 0.f;
-    for (int d = lane; d < W; d += kWave) acc = fmaf(Elem<T>::load(row + d), r[d], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) score[e] = 1.f / (1.f + expf(-acc));
+  constexpr int V = Vec<T>::N;
+  const bool wide = W % V == 0 && (reinterpret_cast<uintptr_t>(h) % 16 == 0) && (reinterpret_cast<uintptr_t>(router) % 16 == 0);
+  for (int e = 0; e < E; e += 2) {
+    // two experts at a time; the sums run over k in the same order whichever path loads them
+    const float* r0 = router + (size_t)e * W;
+    const float* r1 = router + (size_t)min(e + 1, E - 1) * W;
+    float a0 = 0.f, a1 = 0.f;
+    if (wide) {
+      for (int d = lane * V; d < W; d += kWave * V) {
+        float x[V];
+        Vec<T>::load(row + d, x);
+#pragma unroll
+        for (int i = 0; i < V; i += 4) {
+          const float4 p = *reinterpret_cast<const float4*>(r0 + d + i), q = *reinterpret_cast<const float4*>(r1 + d + i);
+          a0 = fmaf(x[i], p.x, a0); a0 = fmaf(x[i + 1], p.y, a0); a0 = fmaf(x[i + 2], p.z, a0); a0 = fmaf(x[i + 3], p.w, a0);
+          a1 = fmaf(x[i], q.x, a1); a1 = fmaf(x[i + 1], q.y, a1); a1 = fmaf(x[i + 2], q.z, a1); a1 = fmaf(x[i + 3], q.w, a1);
+        }
+      }
+    } else {
+      for (int d = lane; d < W; d += kWave) {
+        const float x = Elem<T>::load(row + d);
+        a0 = fmaf(x, r0[d], a0);
+        a1 = fmaf(x, r1[d], a1);
+      }
+    }
+    a0 = wave_sum(a0);
+    a1 = wave_sum(a1);
+    if (lane == 0) {
+      score[e] = 1.f / (1.f + expf(-a0));
+      if (e + 1 < E) score[e + 1] = 1.f / (1.f + expf(-a1));
+    }
   }
   wave_lds_sync();
   // the largest `top` scores, one after the other; a lane looks at the experts lane, lane + 64, ...
@@ -147,51 +181,206 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(
   }
 }
 
-// out[n, c] = sum over the token's chosen experts, in list order, of Wd[e][c] . a[p]; down [E][W][F];
-// out float32.  grid (tokens, slabs of columns).
+// out[k][n][c] = Wd[e][c] . a[p] for the pair p = n top + k and its expert e; down [E][W][F]; out
+// float32 [top][N][W], whose `top` layers the next kernel adds in order.  grid (pairs, slabs of columns).
+constexpr int kDownRows = 16;      // weight rows a wave of the second product walks at once
+
 template <typename T, bool WIDE>
 __global__ __launch_bounds__(256) void moe_down_kernel(
     const T* __restrict__ act, const T* __restrict__ down, const int* __restrict__ chosen,
-    float* __restrict__ out, int W, int F, int top, int slab) {
-  extern __shared__ float x[];         // [top][F]
-  const int n = blockIdx.x;
+    float* __restrict__ out, int N, int W, int F, int top, int slab) {
+  extern __shared__ float x[];         // [F]
+  const int p = blockIdx.x;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
-  for (int d = threadIdx.x; d < top * F; d += blockDim.x) x[d] = Elem<T>::load(act + (size_t)n * top * F + d);
+  for (int d = threadIdx.x; d < F; d += blockDim.x) x[d] = Elem<T>::load(act + (size_t)p * F + d);
   __syncthreads();
   constexpr int V = WIDE ? Vec<T>::N : 1;
+  const T* wd = down + (size_t)chosen[p] * W * F;
+  float* dst = out + ((size_t)(p % top) * N + p / top) * W;
   const int c_end = min(W, (int)(blockIdx.y + 1) * slab);
-  for (int c0 = blockIdx.y * slab + wave * kRows; c0 < c_end; c0 += nwaves * kRows) {
-    float total[kRows];
+  for (int c0 = blockIdx.y * slab + wave * kDownRows; c0 < c_end; c0 += nwaves * kDownRows) {
+    float acc[kDownRows];
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) total[r] = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const T* wd = down + (size_t)chosen[(size_t)n * top + k] * W * F;
-      const float* xk = x + (size_t)k * F;
-      float acc[kRows];
+    for (int r = 0; r < kDownRows; ++r) acc[r] = 0.f;
+    for (int d = lane * V; d < F; d += kWave * V) {
+      float xv[V];
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) acc[r] = 0.f;
-      for (int d = lane * V; d < F; d += kWave * V) {
-        float xv[V];
+      for (int i = 0; i < V; ++i) xv[i] = x[d + i];
 #pragma unroll
-        for (int i = 0; i < V; ++i) xv[i] = xk[d + i];
+      for (int r = 0; r < kDownRows; ++r) {
+        const int c = min(c0 + r, W - 1);
+        float a[V];
+        load_piece<T, WIDE>(wd + (size_t)c * F + d, a);
 #pragma unroll
-        for (int r = 0; r < kRows; ++r) {
-          const int c = min(c0 + r, W - 1);
-          float a[V];
-          load_piece<T, WIDE>(wd + (size_t)c * F + d, a);
-#pragma unroll
-          for (int i = 0; i < V; ++i) acc[r] = fmaf(a[i], xv[i], acc[r]);
-        }
+        for (int i = 0; i < V; ++i) acc[r] = fmaf(a[i], xv[i], acc[r]);
       }
-#pragma unroll
-      for (int r = 0; r < kRows; ++r) total[r] += wave_sum(acc[r]);
     }
-    if (lane < kRows && c0 + lane < c_end) {
+#pragma unroll
+    for (int r = 0; r < kDownRows; ++r) acc[r] = wave_sum(acc[r]);
+    if (lane < kDownRows && c0 + lane < c_end) {
       float v = 0.f;
 #pragma unroll
-      for (int r = 0; r < kRows; ++r)
-        if (r == lane) v = total[r];
-      out[(size_t)n * W + c0 + lane] = v;
+      for (int r = 0; r < kDownRows; ++r)
+        if (r == lane) v = acc[r];
+      dst[c0 + lane] = v;
+    }
+  }
+}
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+};
+
+constexpr int kTilePairs = 64;      // pairs of one expert a block takes
+constexpr int kSortThreads = 1024;
+
+// One block: counts the pairs of every expert, lists the pairs expert by expert (order), and cuts
+// every expert's list into tiles.  Which place a pair gets inside its expert's list depends on the
+// order of LDS atomics; no result depends on it (a pair's products are its own).
+__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
+    const int* __restrict__ chosen, int P, int E, int* __restrict__ order, int* __restrict__ tile_expert,
+    int* __restrict__ tile_start, int* __restrict__ tile_count, int* __restrict__ num_tiles) {
+  extern __shared__ int sort_lds[];     // count [E], first [E + 1], cursor [E]
+  int* count = sort_lds;
+  int* first = count + E;
+  int* cursor = first + E + 1;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = cursor[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&count[chosen[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      first[e] = at;
+      for (int t = 0; t < count[e]; t += kTilePairs) {
+        tile_expert[tiles] = e;
+        tile_start[tiles] = at + t;
+        tile_count[tiles] = min(kTilePairs, count[e] - t);
+        ++tiles;
+      }
+      at += count[e];
+    }
+    first[E] = at;
+    *num_tiles = tiles;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = chosen[p];
+    order[first[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+}
+
+// A block: tile blockIdx.x (up to 16 MT pairs of one expert) and output channels
+// [128 blockIdx.y, +128), a wave 32 of them.  D[channel][pair] accumulates over K in steps of 32;
+// lane (r, kb) holds the weights' row r and the pair r of a tile of 16, 8 consecutive k each.
+// GATED: weights [E][2 R][K], an expert's gate rows then its up rows; a pair's activations are the
+//   row of its token in x; out (bfloat16 [P][R]) = silu(w g) * (w u) with the pair's weight w.
+// else: weights [E][R][K]; a pair's activations are its own row of x; out (float32
+//   [top][N][R]) takes the pair (n, k)'s products at [k][n].
+template <int MT, bool GATED>
+__global__ __launch_bounds__(256) void moe_grouped_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ weights, const int* __restrict__ order,
+    const int* __restrict__ tile_expert, const int* __restrict__ tile_start, const int* __restrict__ tile_count,
+    const int* __restrict__ num_tiles, const float* __restrict__ pair_weight, void* __restrict__ out,
+    int N, int top, int R, int K) {
+  if ((int)blockIdx.x >= *num_tiles) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kb = lane >> 4;
+  const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x], cnt = tile_count[blockIdx.x];
+  const int c0 = blockIdx.y * 128 + wave * 32;
+  if (c0 >= R) return;
+  constexpr int NT = 2;
+  constexpr int WT = GATED ? 2 * NT : NT;       // weight fragments a step: gate and up, or down
+  const bf16_t* base = weights + (size_t)e * (GATED ? 2 : 1) * R * K;
+  const bf16_t* wp[WT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int row = min(c0 + t * 16 + r, R - 1);
+    wp[t] = base + (size_t)row * K + kb * 8;
+    if (GATED) wp[NT + t] = base + (size_t)(R + row) * K + kb * 8;
+  }
+  int pair[MT];
+  const bf16_t* ap[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    pair[t] = order[start + min(t * 16 + r, cnt - 1)];
+    ap[t] = x + (size_t)(GATED ? pair[t] / top : pair[t]) * K + kb * 8;
+  }
+  float4v acc[WT][MT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  const int whole = K / 32;
+  int s = 0;
+  for (; s + 2 <= whole; s += 2) {
+    Frag8 wf[2][WT], af[2][MT];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int t = 0; t < WT; ++t) wf[u][t].u = *reinterpret_cast<const uint4*>(wp[t] + (s + u) * 32);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) af[u][t].u = *reinterpret_cast<const uint4*>(ap[t] + (s + u) * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][i].v, af[u][j].v, acc[i][j], 0, 0, 0);
+  }
+  // leftover steps, the last of which may reach past K (K is a multiple of 8, so a 16-byte piece is
+  // whole or absent; an absent piece is read at k = 0 and zeroed)
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (; s * 32 < K; ++s) {
+    const bool kok = s * 32 + kb * 8 < K;
+    const int koff = kok ? s * 32 : -kb * 8;
+    Frag8 wf[WT], af[MT];
+#pragma unroll
+    for (int t = 0; t < WT; ++t) {
+      const uint4 v = *reinterpret_cast<const uint4*>(wp[t] + koff);
+      wf[t].u = kok ? v : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const uint4 v = *reinterpret_cast<const uint4*>(ap[t] + koff);
+      af[t].u = kok ? v : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, af[j].v, acc[i][j], 0, 0, 0);
+  }
+
+  // acc[i][j][q] = D[channel c0 + i * 16 + kb * 4 + q][pair j * 16 + r]
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    if (j * 16 + r >= cnt) continue;
+    const int p = pair[j];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      const int c = c0 + i * 16 + kb * 4;
+      if (c >= R) continue;
+      if (GATED) {
+        const float w = pair_weight[p];
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float g = acc[i][j][q] * w, u = acc[NT + i][j][q] * w;
+          v[q] = g / (1.f + expf(-g)) * u;
+        }
+        bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)p * R + c;
+        store_four<bf16_t>(dst, v[0], v[1], v[2], v[3], R - c, R % 4 == 0);
+      } else {
+        float* dst = reinterpret_cast<float*>(out) + ((size_t)(p % top) * N + p / top) * R + c;
+        store_four<float>(dst, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3], R - c, R % 4 == 0);
+      }
     }
   }
 }
@@ -249,15 +438,17 @@ TK_API int tk_moe_gate_up(int dtype, const void* h, const void* gate_up, const i
   return launch_status();
 }
 
-// out[N, W] float32 = sum over each token's chosen experts of down[e] act[pair]
+// out[top][N][W] float32: layer k holds down[e] act[pair] of every token's k-th chosen expert
 TK_API int tk_moe_down(int dtype, const void* act, const void* down, const int* chosen, float* out, int N, int W,
                        int F, int top, hipStream_t stream) {
   if (N <= 0) return 0;
   const bool wide = F % (dtype == 0 ? 4 : 8) == 0;
-  if ((size_t)top * F * 4 > 96 * 1024) return -1;
-  const int slab = slab_for(W, N);
-  const dim3 grid(N, (W + slab - 1) / slab);
-  const size_t lds = (size_t)top * F * sizeof(float);
+  if ((size_t)F * 4 > 96 * 1024) return -1;
+  const long want = (1024 + (long)N * top - 1) / ((long)N * top);
+  long slab = (W + want - 1) / want;
+  slab = (slab + 4 * kDownRows - 1) / (4 * kDownRows) * (4 * kDownRows);
+  const dim3 grid(N * top, (unsigned)((W + slab - 1) / slab));
+  const size_t lds = (size_t)F * sizeof(float);
 #define TK_DN(T_, WIDE_)                                                                               \
   {                                                                                                    \
     static bool allowed = false;                                                                       \
@@ -267,7 +458,8 @@ TK_API int tk_moe_down(int dtype, const void* act, const void* down, const int* 
       if (err != hipSuccess) return (int)err;                                                          \
       allowed = true;                                                                                  \
     }                                                                                                  \
-    moe_down_kernel<T_, WIDE_><<<grid, 256, lds, stream>>>((const T_*)act, (const T_*)down, chosen, out, W, F, top, slab); \
+    moe_down_kernel<T_, WIDE_><<<grid, 256, lds, stream>>>((const T_*)act, (const T_*)down, chosen, out, N, W, F, top, \
+                                                           (int)slab);                                 \
   }
   if (dtype == 0 && wide) TK_DN(float, true)
   else if (dtype == 0) TK_DN(float, false)
@@ -277,6 +469,47 @@ TK_API int tk_moe_down(int dtype, const void* act, const void* down, const int* 
   return launch_status();
 }
 
+// The pairs of `chosen` [P] listed expert by expert and cut into tiles of up to 64: order [P],
+// tile_expert / tile_start / tile_count [P / 64 + E], num_tiles [1].
+TK_API int tk_moe_sort(const int* chosen, int P, int E, int* order, int* tile_expert, int* tile_start,
+                       int* tile_count, int* num_tiles, hipStream_t stream) {
+  if (P <= 0) return 0;
+  if (E < 1 || (size_t)(3 * E + 1) * 4 > 60 * 1024) return -1;
+  moe_sort_kernel<<<1, kSortThreads, (size_t)(3 * E + 1) * sizeof(int), stream>>>(chosen, P, E, order, tile_expert, tile_start,
+                                                                                 tile_count, num_tiles);
+  return launch_status();
+}
+
+// bfloat16 only.  gated != 0: x [N][K] the tokens' rows, weights [E][2 R][K], out bfloat16 [N top][R];
+// gated == 0: x [N top][K] the pairs' rows, weights [E][R][K], out float32 [top][N][R].
+// max_tiles: the length of the tile lists (blocks past num_tiles leave at once).
+TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const int* order, const int* tile_expert,
+                          const int* tile_start, const int* tile_count, const int* num_tiles, const float* pair_weight,
+                          void* out, int N, int top, int R, int K, int max_tiles, int rows_hint, hipStream_t stream) {
+  if (N <= 0 || max_tiles <= 0) return 0;
+  if (K % 8 != 0 || K < 8 || R < 1 || (uintptr_t)x % 16 != 0 || (uintptr_t)weights % 16 != 0) return -1;
+  const dim3 grid(max_tiles, (R + 127) / 128);
+#define TK_GROUPED(MT_)                                                                                           \
+  {                                                                                                               \
+    if (gated)                                                                                                    \
+      moe_grouped_kernel<MT_, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order,    \
+                                                              tile_expert, tile_start, tile_count, num_tiles,     \
+                                                              pair_weight, out, N, top, R, K);                    \
+    else                                                                                                          \
+      moe_grouped_kernel<MT_, false><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order,   \
+                                                               tile_expert, tile_start, tile_count, num_tiles,    \
+                                                               pair_weight, out, N, top, R, K);                   \
+  }
+  // rows_hint: the most pairs an expert can have (the step's pairs): tiles are never fuller than that
+  if (rows_hint <= 16) TK_GROUPED(1)
+  else if (rows_hint <= 32) TK_GROUPED(2)
+  else TK_GROUPED(4)
+#undef TK_GROUPED
+  return launch_status();
+}
+
 TK_SLOTS(tk_moe_route)
 TK_SLOTS(tk_moe_gate_up)
 TK_SLOTS(tk_moe_down)
+TK_SLOTS(tk_moe_sort)
+TK_SLOTS(tk_moe_grouped)

@@ -216,6 +216,9 @@ _SIGS = {
         "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "tk_moe_gate_up": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "tk_moe_down": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "tk_moe_sort": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+        "tk_moe_grouped": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "gemm_tiled": {
         "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
@@ -833,16 +836,69 @@ def moe_gate_up(h: torch.Tensor, gate_up: torch.Tensor, chosen: torch.Tensor, we
 
 
 def moe_down(act: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, out: torch.Tensor, top: int) -> None:
-    """out[n] = sum over the token's chosen experts, in list order, of down_e act[n * top + k]; out float32 [N, width]."""
+    """out[k, n] = down_e act[n * top + k] for the token's k-th chosen expert e; out float32 [top, N, width]:
+    partial sums that the next kernel adds in order."""
     _gpu(act, down, chosen, out)
     e, w, f = down.shape
-    n = out.shape[0]
-    _need(act.shape == (n * top, f) and act.dtype == down.dtype and out.dtype == torch.float32 and out.shape == (n, w),
+    n = out.shape[1]
+    _need(act.shape == (n * top, f) and act.dtype == down.dtype and out.dtype == torch.float32 and out.shape == (top, n, w),
           "expert outputs do not match")
-    _need(top * f * 4 <= MOE_LDS_BYTES, "a token's expert activations must fit LDS")
+    _need(f * 4 <= MOE_LDS_BYTES, "a row of expert activations must fit LDS")
     _note(f"{n}x{top} {w}x{f}", min(n * top, e) * w * f * act.element_size(), 2.0 * n * top * w * f)
     _check(_fn("moe", "tk_moe_down")(_code(act.dtype), _p(act), _p(down), _p(chosen), _p(out), n, w, f, top, _stream()),
            "moe_down")
+
+
+MOE_TILE_PAIRS = 64        # pairs of one expert that a block of the grouped products takes (csrc/moe.hip: kTilePairs)
+MOE_GROUPED_FROM = 65      # pairs of a step from which the experts' products run grouped on the matrix cores
+
+
+def moe_grouped_fits(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, pairs: int) -> bool:
+    """Whether a step's expert products take the grouped form: bfloat16, enough pairs, rows that
+    fill 16-byte pieces, and few enough experts for the one block that lists the pairs."""
+    f = down.shape[2]
+    return (h.dtype == torch.bfloat16 and pairs >= MOE_GROUPED_FROM and h.shape[1] % 8 == 0 and f % 8 == 0
+            and gate_up.shape[0] <= 4096)
+
+
+def moe_sort(chosen: torch.Tensor, num_experts: int):
+    """The step's (token, expert) pairs listed expert by expert and cut into tiles of up to
+    ``MOE_TILE_PAIRS``: (order, tile_expert, tile_start, tile_count, num_tiles) int32 on the device."""
+    _gpu(chosen)
+    pairs = chosen.numel()
+    max_tiles = pairs // MOE_TILE_PAIRS + num_experts
+    lists = torch.empty(pairs + 3 * max_tiles + 1, dtype=torch.int32, device=chosen.device)
+    order, rest = lists[:pairs], lists[pairs:]
+    tile_expert, tile_start, tile_count = (rest[i * max_tiles:(i + 1) * max_tiles] for i in range(3))
+    num_tiles = rest[3 * max_tiles:]
+    _need(chosen.dtype == torch.int32, "lists of chosen experts are int32")
+    _check(_fn("moe", "tk_moe_sort")(_p(chosen), pairs, num_experts, _p(order), _p(tile_expert), _p(tile_start),
+                                     _p(tile_count), _p(num_tiles), _stream()), "moe_sort")
+    return order, tile_expert, tile_start, tile_count, num_tiles
+
+
+def moe_grouped(x: torch.Tensor, weights: torch.Tensor, lists: tuple, pair_weight: torch.Tensor | None,
+                out: torch.Tensor, *, tokens: int, top: int, gated: bool) -> None:
+    """One of the experts' two products over the tiles of ``lists`` (``moe_sort``), bfloat16 on the matrix
+    cores.  ``gated``: x [tokens, K] the tokens' rows, weights [E, 2 R, K] (gate rows, then up rows), out
+    bfloat16 [tokens * top, R] = silu(w g) * (w u) with the pairs' weights w.  Else: x [tokens * top, K] the
+    pairs' rows, weights [E, R, K], out float32 [top, tokens, R]."""
+    order, tile_expert, tile_start, tile_count, num_tiles = lists
+    _gpu(x, weights, pair_weight, out)
+    k = x.shape[1]
+    e = weights.shape[0]
+    r = weights.shape[1] // (2 if gated else 1)
+    _need(x.dtype == weights.dtype == torch.bfloat16 and weights.shape[2] == k and k % 8 == 0, "grouped expert products are bfloat16 with rows of 16-byte pieces")
+    _need(order.numel() == tokens * top and x.shape[0] == (tokens if gated else tokens * top), "the pairs' list does not match")
+    if gated:
+        _need(out.dtype == torch.bfloat16 and out.shape == (tokens * top, r) and pair_weight is not None
+              and pair_weight.dtype == torch.float32 and pair_weight.numel() >= tokens * top, "gated output does not match")
+    else:
+        _need(out.dtype == torch.float32 and out.shape == (top, tokens, r), "the pairs' outputs are float32 [top, tokens, width]")
+    _note(f"{tokens}x{top} {weights.shape[1]}x{k}", min(tokens * top, e) * weights.shape[1] * k * 2, 2.0 * tokens * top * weights.shape[1] * k)
+    _check(_fn("moe", "tk_moe_grouped")(
+        int(gated), _p(x), _p(weights), _p(order), _p(tile_expert), _p(tile_start), _p(tile_count), _p(num_tiles),
+        _p(pair_weight), _p(out), tokens, top, r, k, tile_expert.numel(), tokens * top, _stream()), "moe_grouped")
 
 
 FEWROWS_MAX_ROWS = 64          # float32 products of up to this many rows stream the weights, a lane a weight row,

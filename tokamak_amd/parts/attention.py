@@ -176,6 +176,9 @@ class RotatedUnitAttention(Mixer):
     def pair_flops(self) -> float:
         return 2.0 * self.num_heads * (self.head_dim + self.value_dim)
 
+    def visible_keys(self, position: int) -> int:
+        return position + 1 if self.chunk is None else position % self.chunk + 1
+
     def forward(self, h, batch, store, writes_cache: bool = True, position: PositionData | None = None):
         nh, nkv, hd, vd = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
         n = h.shape[0]

@@ -82,6 +82,12 @@ class Part:
         """The planner of the work lists this part's kernels read, or None."""
         return None
 
+    def matrix_share(self, tokens: int) -> tuple[float, float]:
+        """For the measurement's count of a step's work: (the share of the part's matrix elements
+        that one token is multiplied with, the share that a step of ``tokens`` tokens reads).  Both
+        1 unless the part chooses among its matrices token by token."""
+        return 1.0, 1.0
+
     def check_page_size(self, page_size: int) -> None:
         """Raise ``ValueError`` if the part's kernels cannot work with cache pages of
         ``page_size`` tokens."""
@@ -187,6 +193,10 @@ class Mixer(Part):
         call, for the measurement's count of a step's work; 0 for a mixer whose work does
         not grow with the context."""
         return 0.0
+
+    def visible_keys(self, position: int) -> int:
+        """How many cached positions (its own included) the token at ``position`` reads."""
+        return position + 1
 
     def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True,
                 position: PositionData | None = None) -> torch.Tensor:

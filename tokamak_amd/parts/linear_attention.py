@@ -74,7 +74,10 @@ class GatedLinearAttention(Mixer):
         # (split products leave float32 partial sums, which the scan adds as it loads)
         q, k, v, gate = (linear(h, w, allow_partials=True) for w in (self.q, self.k, self.v, self.g))
         low = linear(h, self.a1)
-        decay_in = linear(low, self.a2, out_dtype=torch.float32, allow_partials=True)
+        # (few rows: float32 or split partial sums from the streaming product; a long portion: the
+        # library's product in the compute dtype, as for the other projections)
+        few = n <= ops.STREAM_MAX_ROWS
+        decay_in = linear(low, self.a2, out_dtype=torch.float32 if few else None, allow_partials=True)
         out = torch.empty((n, self.num_heads * self.value_dim), dtype=self.dtype, device=h.device)
         ops.gla_scan(q, k, v, gate, decay_in, self.bias, self.gain, store.state["S"], out, batch,
                      heads=self.num_heads, dim=self.head_dim, vdim=self.value_dim,

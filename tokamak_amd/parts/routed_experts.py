@@ -56,14 +56,28 @@ class RoutedExperts(FeedForward):
         self.gate_up = torch.stack([torch.cat([fetch(b + gate), fetch(b + up)], dim=0) for b in bases]).contiguous()
         self.down = torch.stack([fetch(b + down) for b in bases]).contiguous()
 
+    def matrix_share(self, tokens: int) -> tuple[float, float]:
+        e, top = self.num_experts, self.top
+        router, expert = e * self.hidden_size, 3 * self.intermediate_size * self.hidden_size
+        met = e * (1.0 - (1.0 - top / e) ** max(tokens, 0))     # experts that a step of so many tokens meets, on average
+        return (router + top * expert) / (router + e * expert), (router + met * expert) / (router + e * expert)
+
     def forward(self, h, batch):
+        """Float32 partial sums [top, N, width]: layer k holds every token's k-th chosen expert's output;
+        whoever adds the sub-layer's output to the stream sums them in that order."""
         n, top = h.shape[0], self.top
         chosen = torch.empty((n, top), dtype=torch.int32, device=h.device)
         weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
         ops.moe_route(h, self.router, chosen, weight, top)
         act = torch.empty((n * top, self.intermediate_size), dtype=h.dtype, device=h.device)
+        out = torch.empty((top, n, self.hidden_size), dtype=torch.float32, device=h.device)
+        if ops.moe_grouped_fits(h, self.gate_up, self.down, n * top):
+            # many tokens: the pairs listed expert by expert, tiles of one expert on the matrix cores
+            lists = ops.moe_sort(chosen, self.num_experts)
+            ops.moe_grouped(h, self.gate_up, lists, weight, act, tokens=n, top=top, gated=True)
+            ops.moe_grouped(act, self.down, lists, None, out, tokens=n, top=top, gated=False)
+            return out
         ops.moe_gate_up(h, self.gate_up, chosen, weight, act, top)
-        out = torch.empty((n, self.hidden_size), dtype=torch.float32, device=h.device)
         ops.moe_down(act, self.down, chosen, out, top)
         return out
 
