@@ -180,8 +180,9 @@ def test_gated_linear_attention_alone_in_portions_and_slots(dtype, heads, dim, v
                                dict(heads=2, kv_heads=2, dim=40, vdim=16, chunk=33, rot=0),
                                dict(heads=8, kv_heads=2, dim=128, vdim=128, chunk=16, rot=64, base=1e5),
                                dict(heads=2, kv_heads=1, dim=64, vdim=64, chunk=None, rot=32),
-                               dict(heads=2, kv_heads=1, dim=16, vdim=16, chunk=1, rot=2)],
-                         ids=["g2", "g3", "g1", "wide", "full", "one"])
+                               dict(heads=2, kv_heads=1, dim=16, vdim=16, chunk=1, rot=2),
+                               dict(heads=4, kv_heads=1, dim=64, vdim=64, chunk=50, rot=64)],
+                         ids=["g2", "g3", "g1", "wide", "full", "one", "mid"])
 def test_chunked_attention_alone(dtype, a):
     """A portion from position zero, one that ends inside a page and inside a chunk, two tokens, then
     single tokens; the request's pages scattered; the position that starts a chunk given a key that
@@ -189,7 +190,8 @@ def test_chunked_attention_alone(dtype, a):
     from tokamak_amd.config import get_part
     from tokamak_amd.engine.storage import SlotStore
 
-    width, eps, page = 64, 1e-5, 8
+    width, eps = 64, 1e-5
+    page = 16 if a["dim"] >= 64 else 8       # (heads of 64 and 128 with pages of 16: the matrix-core kernel for portions in bfloat16)
     cfg = model_json([attention(**a)], width=width, eps=eps)
     m = cfg["layers"][0]["mixer"]
     w = random_weights(cfg, seed=a["dim"])

@@ -487,7 +487,7 @@ void attention_prefill_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit,
-    int split_keys, int num_items, int nh, int nkv, int ps, float scale_log2) {
+    int split_keys, int num_items, int nh, int nkv, int ps, float scale_log2, int chunk) {
   constexpr int KCH = HD / 32, DBL = HD / 16;
   constexpr int THREADS = kPrefillThreads;
   constexpr int GROUP_PIECES = 2 * HD;         // 16-byte pieces of K (and of V) per 16-key group
@@ -519,9 +519,14 @@ void attention_prefill_kernel(
   // With several splits (few tiles over a long context) this block takes the keys
   // [k_begin, k_begin + split_keys), a multiple of 64, and writes an unnormalised partial.
   const int split = blockIdx.z;
-  const int k_begin = split * split_keys;
+  // chunk > 0 (only without splits): a query sees the keys of its own chunk of that many positions
+  // only, chunks counted from position 0.  The walk starts at the stage that holds the first key
+  // the tile's first query sees; what a column's own chunk does not hold is masked below.
+  const int c_first = chunk > 0 ? c_pos - c_pos % chunk : 0;
+  const int first_of_last = chunk > 0 ? last_pos - last_pos % chunk : 0;
+  const int k_begin = chunk > 0 ? (pos0 - pos0 % chunk) & ~63 : split * split_keys;
   if (k_begin > last_pos) return;  // no key of this tile lies in the split (the whole block leaves)
-  const int last_key = min(last_pos, k_begin + split_keys - 1);
+  const int last_key = chunk > 0 ? last_pos : min(last_pos, k_begin + split_keys - 1);
 
   bf16x8 qreg[KCH];
   {
@@ -635,13 +640,13 @@ void attention_prefill_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) sv[j][i] = sc[i];
     }
-    if (s0 + 63 > pos0) {  // some key of this stage is hidden from some column, or is past the end
+    if (s0 + 63 > pos0 || s0 < first_of_last) {  // some key of this stage is hidden from some column, or is past the end
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = s0 + j * 16 + kb * 4 + i;
-          if (key > c_pos || key > last_pos) sv[j][i] = -INFINITY;
+          if (key > c_pos || key > last_pos || key < c_first) sv[j][i] = -INFINITY;
         }
     }
     float tmax = -INFINITY;
@@ -1273,13 +1278,13 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
                           const int* block_tables, int max_pages, const int* positions,
                           const int* req_of_token, const int* item_token, const int* item_count,
                           int num_items, void* out, float* part_o, float* part_ml, int nsplit,
-                          int split_keys, int nh, int nkv, int ps, float scale, hipStream_t stream) {
+                          int split_keys, int nh, int nkv, int ps, float scale, hipStream_t stream, int chunk) {
   const int G = nh / nkv;
   dim3 grid(nkv * (G / HPB), num_items, nsplit);
   attention_prefill_kernel<HD, HPB, OCC><<<grid, kPrefillThreads, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
-      split_keys, num_items, nh, nkv, ps, scale * 1.4426950408889634f);
+      split_keys, num_items, nh, nkv, ps, scale * 1.4426950408889634f, chunk);
   if (nsplit > 1) {
     dim3 mgrid(num_items * 16, nh);
     attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, item_count,
@@ -1415,10 +1420,12 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
                              const int* block_tables, int max_pages, const int* positions,
                              const int* req_of_token, const int* item_token, const int* item_count,
                              int num_items, void* out, float* part_o, float* part_ml, int nsplit,
-                             int split_keys, int nh, int nkv, int hd, int ps, float scale,
+                             int split_keys, int nh, int nkv, int hd, int ps, float scale, int chunk,
                              hipStream_t stream) {
   if (num_items <= 0) return 0;
   if (mode < 0 || mode > 4) return -1;
+  // chunked visibility: the narrow form for tiles only, their keys not split over blocks
+  if (chunk < 0 || (chunk > 0 && ((mode != 1 && mode != 2) || nsplit != 1))) return -1;
   if (nkv <= 0 || nh % nkv != 0 || ps < 16 || (ps & (ps - 1)) != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
   if (num_items > 65535 || nh > 65535) return -1;
   const int G = nh / nkv;
@@ -1463,7 +1470,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
   if (nsplit > 1 && (split_keys % 64 != 0 || (long)num_items * 16 > 65535)) return -1;
 #define TK_PARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
-      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, chunk
   const bool dense = mode == 2;
   if (hd == 128) {
     if (hpb == 4) return dense ? launch_prefill<128, 4, 4>(TK_PARGS) : launch_prefill<128, 4, 2>(TK_PARGS);

@@ -28,7 +28,7 @@ using namespace tk;
 
 namespace {
 
-constexpr int kRouteWaves = 4;     // tokens a block of the router takes, a wave each
+constexpr int kRouteWaves = 8;     // waves of a block of the router, which share a token's experts
 constexpr int kRows = 8;           // weight rows a wave walks at once
 
 template <typename T> struct Vec;
@@ -52,21 +52,20 @@ template <> struct Vec<bf16_t> {
   }
 };
 
-// A wave a token: lanes stride the width, one expert after the other.
+// A block a token: its waves take the experts two at a time (lanes stride the width), then the
+// first wave picks the largest scores.
 template <typename T>
 __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
     const T* __restrict__ h, const float* __restrict__ router, int* __restrict__ chosen,
     float* __restrict__ weight, int N, int W, int E, int top) {
-  extern __shared__ float lds[];       // [kRouteWaves][E]
+  extern __shared__ float score[];     // [E]
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int n = blockIdx.x * kRouteWaves + wave;
-  if (n >= N) return;                  // nothing below synchronises across waves
-  float* score = lds + (size_t)wave * E;
+  const int n = blockIdx.x;
   const T* row = h + (size_t)n * W;
   constexpr int V = Vec<T>::N;
   const bool wide = W % V == 0 && (reinterpret_cast<uintptr_t>(h) % 16 == 0) && (reinterpret_cast<uintptr_t>(router) % 16 == 0);
-  for (int e = 0; e < E; e += 2) {
-    // two experts at a time; the sums run over k in the same order whichever path loads them
+  for (int e = 2 * wave; e < E; e += 2 * kRouteWaves) {
+    // the sums run over k in the same order whichever path loads them
     const float* r0 = router + (size_t)e * W;
     const float* r1 = router + (size_t)min(e + 1, E - 1) * W;
     float a0 = 0.f, a1 = 0.f;
@@ -95,7 +94,8 @@ __global__ __launch_bounds__(kRouteWaves * kWave) void moe_route_kernel(
       if (e + 1 < E) score[e + 1] = 1.f / (1.f + expf(-a1));
     }
   }
-  wave_lds_sync();
+  __syncthreads();
+  if (wave != 0) return;
   // the largest `top` scores, one after the other; a lane looks at the experts lane, lane + 64, ...
   for (int k = 0; k < top; ++k) {
     float best = -1.f;
@@ -273,8 +273,8 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
   }
 }
 
-// A block: tile blockIdx.x (up to 16 MT pairs of one expert) and output channels
-// [128 blockIdx.y, +128), a wave 32 of them.  D[channel][pair] accumulates over K in steps of 32;
+// A block: tile blockIdx.x (up to 16 MT pairs of one expert) and four waves' output channels, a
+// wave 32 of them (64 where there is no gate: as many products a load).  D[channel][pair] accumulates over K in steps of 32;
 // lane (r, kb) holds the weights' row r and the pair r of a tile of 16, 8 consecutive k each.
 // GATED: weights [E][2 R][K], an expert's gate rows then its up rows; a pair's activations are the
 //   row of its token in x; out (bfloat16 [P][R]) = silu(w g) * (w u) with the pair's weight w.
@@ -290,9 +290,9 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x], cnt = tile_count[blockIdx.x];
-  const int c0 = blockIdx.y * 128 + wave * 32;
+  constexpr int NT = GATED ? 2 : 4;             // tiles of 16 output channels a wave
+  const int c0 = (blockIdx.y * 4 + wave) * (16 * NT);
   if (c0 >= R) return;
-  constexpr int NT = 2;
   constexpr int WT = GATED ? 2 * NT : NT;       // weight fragments a step: gate and up, or down
   const bf16_t* base = weights + (size_t)e * (GATED ? 2 : 1) * R * K;
   const bf16_t* wp[WT];
@@ -391,9 +391,9 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 TK_API int tk_moe_route(int dtype, const void* h, const float* router, int* chosen, float* weight, int N,
                         int W, int E, int top, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (E < 1 || top < 1 || top > E || W < 1 || (size_t)E * kRouteWaves * 4 > 64 * 1024) return -1;
-  const unsigned blocks = (unsigned)((N + kRouteWaves - 1) / kRouteWaves);
-  const size_t lds = (size_t)kRouteWaves * E * sizeof(float);
+  if (E < 1 || top < 1 || top > E || W < 1 || (size_t)E * 4 > 64 * 1024) return -1;
+  const unsigned blocks = (unsigned)N;
+  const size_t lds = (size_t)E * sizeof(float);
   if (dtype == 0)
     moe_route_kernel<float><<<blocks, kRouteWaves * kWave, lds, stream>>>((const float*)h, router, chosen, weight, N, W, E, top);
   else
@@ -488,7 +488,8 @@ TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const i
                           void* out, int N, int top, int R, int K, int max_tiles, int rows_hint, hipStream_t stream) {
   if (N <= 0 || max_tiles <= 0) return 0;
   if (K % 8 != 0 || K < 8 || R < 1 || (uintptr_t)x % 16 != 0 || (uintptr_t)weights % 16 != 0) return -1;
-  const dim3 grid(max_tiles, (R + 127) / 128);
+  const int channels = gated ? 128 : 256;      // a block's
+  const dim3 grid(max_tiles, (R + channels - 1) / channels);
 #define TK_GROUPED(MT_)                                                                                           \
   {                                                                                                               \
     if (gated)                                                                                                    \

@@ -285,7 +285,9 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     when the tiles are few and the context long.  Everything else, and whatever
     the MFMA library does not instantiate: the generic float32-arithmetic kernel.
     ``value_dim``: size of a value head if not ``head_dim``.  ``chunk``: a query sees the
-    keys of its own chunk of that many positions only (the generic kernel).
+    keys of its own chunk of that many positions only: the tiles of prompt portions on the
+    matrix cores where the shape fits (tiles of 16, walking from the chunk's first stage),
+    single tokens (which read a chunk at most) and everything else in the generic kernel.
     """
     value_dim = head_dim if value_dim is None else value_dim
     work = work_of(batch)
@@ -307,14 +309,28 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
                                  num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale,
                                  note=(decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair) if profiling else None):
             return
+    tiles = (work.tile_first, work.tile_count, work.num_tiles, work.single, work.num_single)
+    if (chunk and work.num_tiles and value_dim == head_dim
+            and mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, None)):
+        if profiling:
+            ops._note(f"portions {work.num_tiles} tiles, chunks of {chunk}", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+        if ops.attention_mfma("tokens", q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token,
+                              work.tile_first, work.tile_count, work.num_tiles, out, num_heads=num_heads,
+                              num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale, chunk=chunk):
+            if profiling and work.num_single:
+                ops._note(f"{work.num_single} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
+            ops.paged_attention_generic(
+                q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
+                num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
+                scale=scale, value_dim=value_dim, chunk=chunk, tiles=tiles, only_single=True)
+            return
     if profiling:
         ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,
                   (decode_keys + tile_pairs) * flops_per_pair)
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-        scale=scale, window=window, value_dim=value_dim, chunk=chunk,
-        tiles=(work.tile_first, work.tile_count, work.num_tiles, work.single, work.num_single))
+        scale=scale, window=window, value_dim=value_dim, chunk=chunk, tiles=tiles)
 
 
 def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *, num_heads, num_kv_heads,

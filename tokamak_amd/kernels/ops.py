@@ -253,7 +253,7 @@ _SIGS = {
     "attention_mfma": {
         "tk_attention_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                              c_int, c_int, c_int, c_int, c_float, c_void_p],
+                              c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     },
     "attention_fused": {
         "tk_attention_decode_fused": [c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
@@ -1232,7 +1232,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             num_kv_heads: int, head_dim: int, page_size: int, scale: float,
                             window: int | None = None, tiles: tuple | None = None,
                             share_heads: bool | None = None, value_dim: int | None = None,
-                            chunk: int | None = None) -> None:
+                            chunk: int | None = None, only_single: bool = False) -> None:
     """Causal attention of each query token over its request's pages.  ``tiles``:
     (tile_first, tile_count, num_tiles, single_tokens, num_single), the step's work lists (tiles
     of up to 16 consecutive tokens of one request, and token rows that run alone), which together
@@ -1241,7 +1241,8 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     of a group share a block (and the keys it loads) for the tokens that run alone; None chooses by
     how many there are; the same bits again.  ``value_dim``: size of a value head if it differs from
     ``head_dim``.  ``chunk``: a query sees only the keys of its own chunk of that many positions
-    (counted from position 0); not together with ``window``."""
+    (counted from position 0); not together with ``window``.  ``only_single``: the tokens of the tiles
+    are left to another kernel."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out)
     n = positions.numel()
     vd = head_dim if value_dim is None else int(value_dim)
@@ -1259,7 +1260,14 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
           and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
     tile_first = tile_count = single = None
     num_tiles = num_single = 0
-    if tiles is not None and tiles[2] > 0:
+    if tiles is not None and only_single:
+        if tiles[4] == 0:
+            return
+        # (the list of tiles is there and empty: only the tokens of ``single`` run)
+        tile_first, tile_count, num_tiles, single, num_single = tiles[3], tiles[3], 0, tiles[3], tiles[4]
+        _need(single is not None and single.is_cuda and single.dtype == torch.int32 and single.numel() >= num_single,
+              "bad list of single tokens")
+    elif tiles is not None and tiles[2] > 0:
         tile_first, tile_count, num_tiles, single, num_single = tiles
         _gpu(tile_first, tile_count)
         _need(tile_first.dtype == torch.int32 and tile_count.dtype == torch.int32
@@ -1280,7 +1288,8 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
                    block_tables: torch.Tensor, positions: torch.Tensor, req_of_token: torch.Tensor,
                    item_token: torch.Tensor, item_count: torch.Tensor | None, num_items: int,
                    out: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,
-                   page_size: int, scale: float, split_keys: int = 256, num_splits: int = 1) -> bool:
+                   page_size: int, scale: float, split_keys: int = 256, num_splits: int = 1,
+                   chunk: int | None = None) -> bool:
     """bf16 attention on the matrix cores.  ``mode`` "heads": every item is one
     decode token; "tokens": every item is up to 16 consecutive tokens of one
     request ("tokens_dense": the same, with the kernel variant for tiles that all
@@ -1289,8 +1298,9 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     a kv head and shares of the keys, any group size).  With ``num_splits`` > 1 the keys of an item are cut into pieces of
     ``split_keys`` (a multiple of 16; of 64 in "tokens" mode), each its own block, and a
     second kernel merges the pieces (in "heads" mode the sixteen waves of a block share a piece, so
-    ``split_keys`` is a multiple of 256).  Returns False (nothing launched) if the shape
-    is not instantiated."""
+    ``split_keys`` is a multiple of 256).  ``chunk`` ("tokens" and "tokens_dense" without splits): a
+    query sees the keys of its own chunk of that many positions only.  Returns False (nothing
+    launched) if the shape is not instantiated."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, item_token, item_count, out)
     n = positions.numel()
     _need(q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
@@ -1307,6 +1317,8 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
           "mode is heads, tokens, tokens_dense, tokens_wide or tokens_group")
     _need(mode not in ("tokens_wide", "tokens_group") or num_splits == 1, "the wide and group forms do not split keys over blocks")
     _need(mode != "heads" or num_splits == 1 or split_keys % 256 == 0, "heads mode splits keys in multiples of 256")
+    _need(not chunk or (mode in ("tokens", "tokens_dense") and num_splits == 1 and chunk > 0),
+          "chunked visibility: tiles of 16 tokens, keys not split")
     if mode != "heads":
         _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items,
               "tokens mode needs item counts")
@@ -1321,7 +1333,7 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
         {"heads": 0, "tokens": 1, "tokens_dense": 2, "tokens_wide": 3, "tokens_group": 4}[mode], _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
         block_tables.shape[1], _p(positions), _p(req_of_token), _p(item_token), _p(item_count),
         num_items, _p(out), _p(part_o), _p(part_ml), num_splits, split_keys, num_heads, num_kv_heads,
-        head_dim, page_size, float(scale), _stream())
+        head_dim, page_size, float(scale), int(chunk or 0), _stream())
     if status == NOT_INSTANTIATED:
         return False
     _check(status, "attention_mfma")
