@@ -237,7 +237,8 @@ def clear_of(h, w, top, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-@pytest.mark.parametrize("width,ff,n,top", [(64, 32, 4, 2), (48, 24, 12, 1), (72, 40, 5, 5), (36, 20, 7, 3), (256, 136, 3, 2)])
+@pytest.mark.parametrize("width,ff,n,top", [(64, 32, 4, 2), (48, 24, 12, 1), (72, 40, 5, 5), (36, 20, 7, 3), (256, 136, 3, 2),
+                                            (128, 192, 2, 1)])
 def test_routed_experts_alone(dtype, width, ff, n, top):
     """Numbers of experts that are no power of two, one expert a token, every expert a token, sizes
     that do not fill 16-byte pieces; the rows whose choice of experts is no close call are compared."""
@@ -250,15 +251,16 @@ def test_routed_experts_alone(dtype, width, ff, n, top):
     assert set(part.expected_tensors("l0.mlp.")) == {k for k in w if k.startswith("l0.mlp.")}
     part.bind("l0.mlp.", fetcher(w, dtype))
     g = torch.Generator().manual_seed(3)
-    h = torch.randn(70, width, generator=g).to(dtype)
+    rows = 70 if n > 2 else 500         # (two experts and 500 tokens, K in chunks of 64: full tiles, their activations through LDS)
+    h = torch.randn(rows, width, generator=g).to(dtype)
     want = plain.routed_experts(h.double(), double(w), "l0.mlp.", cfg["layers"][0]["mlp"]).float()
-    got = part.forward(h.to(DEV), make_batch([(70, 0, [0])]))
-    assert got.dtype == torch.float32 and got.shape == (top, 70, width)      # a layer per chosen expert, added by the reader
+    got = part.forward(h.to(DEV), make_batch([(rows, 0, [0])]))
+    assert got.dtype == torch.float32 and got.shape == (top, rows, width)      # a layer per chosen expert, added by the reader
     got = got.sum(0).cpu()
     few = part.forward(h[:9].to(DEV), make_batch([(9, 0, [0])])).sum(0).cpu()   # the form for few tokens
     close(few[clear_of(h[:9], w, top, n)], want[:9][clear_of(h[:9], w, top, n)], dtype)
     clear = clear_of(h, w, top, n)
-    assert int(clear.sum()) >= 60
+    assert int(clear.sum()) >= 0.85 * rows
     close(got[clear], want[clear], dtype)
     # the weight acts on the expert's input: it is not the same as weighting the output
     one = plain.routed_experts(h[:1].double(), double(w), "l0.mlp.", cfg["layers"][0]["mlp"])

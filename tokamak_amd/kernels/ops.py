@@ -216,9 +216,9 @@ _SIGS = {
         "tk_moe_route": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "tk_moe_gate_up": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "tk_moe_down": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-        "tk_moe_sort": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+        "tk_moe_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
         "tk_moe_grouped": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "gemm_tiled": {
         "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
@@ -861,20 +861,21 @@ def moe_grouped_fits(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
             and gate_up.shape[0] <= 4096)
 
 
-def moe_sort(chosen: torch.Tensor, num_experts: int):
+def moe_sort(chosen: torch.Tensor, num_experts: int, tile_pairs: int = MOE_TILE_PAIRS):
     """The step's (token, expert) pairs listed expert by expert and cut into tiles of up to
-    ``MOE_TILE_PAIRS``: (order, tile_expert, tile_start, tile_count, num_tiles) int32 on the device."""
+    ``tile_pairs``: (order, tile_expert, tile_start, tile_count, num_tiles, tile_pairs), int32 on the device."""
     _gpu(chosen)
     pairs = chosen.numel()
-    max_tiles = pairs // MOE_TILE_PAIRS + num_experts
+    _need(tile_pairs == MOE_TILE_PAIRS, "tiles hold 64 pairs")
+    max_tiles = pairs // tile_pairs + num_experts
     lists = torch.empty(pairs + 3 * max_tiles + 1, dtype=torch.int32, device=chosen.device)
     order, rest = lists[:pairs], lists[pairs:]
     tile_expert, tile_start, tile_count = (rest[i * max_tiles:(i + 1) * max_tiles] for i in range(3))
     num_tiles = rest[3 * max_tiles:]
     _need(chosen.dtype == torch.int32, "lists of chosen experts are int32")
-    _check(_fn("moe", "tk_moe_sort")(_p(chosen), pairs, num_experts, _p(order), _p(tile_expert), _p(tile_start),
+    _check(_fn("moe", "tk_moe_sort")(_p(chosen), pairs, num_experts, tile_pairs, _p(order), _p(tile_expert), _p(tile_start),
                                      _p(tile_count), _p(num_tiles), _stream()), "moe_sort")
-    return order, tile_expert, tile_start, tile_count, num_tiles
+    return order, tile_expert, tile_start, tile_count, num_tiles, tile_pairs
 
 
 def moe_grouped(x: torch.Tensor, weights: torch.Tensor, lists: tuple, pair_weight: torch.Tensor | None,
@@ -883,7 +884,7 @@ def moe_grouped(x: torch.Tensor, weights: torch.Tensor, lists: tuple, pair_weigh
     cores.  ``gated``: x [tokens, K] the tokens' rows, weights [E, 2 R, K] (gate rows, then up rows), out
     bfloat16 [tokens * top, R] = silu(w g) * (w u) with the pairs' weights w.  Else: x [tokens * top, K] the
     pairs' rows, weights [E, R, K], out float32 [top, tokens, R]."""
-    order, tile_expert, tile_start, tile_count, num_tiles = lists
+    order, tile_expert, tile_start, tile_count, num_tiles, tile_pairs = lists
     _gpu(x, weights, pair_weight, out)
     k = x.shape[1]
     e = weights.shape[0]
@@ -898,7 +899,7 @@ def moe_grouped(x: torch.Tensor, weights: torch.Tensor, lists: tuple, pair_weigh
     _note(f"{tokens}x{top} {weights.shape[1]}x{k}", min(tokens * top, e) * weights.shape[1] * k * 2, 2.0 * tokens * top * weights.shape[1] * k)
     _check(_fn("moe", "tk_moe_grouped")(
         int(gated), _p(x), _p(weights), _p(order), _p(tile_expert), _p(tile_start), _p(tile_count), _p(num_tiles),
-        _p(pair_weight), _p(out), tokens, top, r, k, tile_expert.numel(), tokens * top, _stream()), "moe_grouped")
+        _p(pair_weight), _p(out), tokens, top, r, k, tile_expert.numel(), tokens * top, tile_pairs, _stream()), "moe_grouped")
 
 
 FEWROWS_MAX_ROWS = 64          # float32 products of up to this many rows stream the weights, a lane a weight row,
