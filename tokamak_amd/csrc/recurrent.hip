@@ -312,17 +312,24 @@ int launch_scan(ScanIn r, ScanIn k, ScanIn v, ScanIn g, ScanIn d, const float* w
 
 struct GlaShape {
   int heads, dim, vdim, columns, slices, slice;   // threads = columns * slices; a thread owns `slice` key channels of a value column
+  int splits;                                     // blocks that share a head's value columns (blockIdx.z), `columns` each
 };
 
-// A block a (request, head).  Thread (ks, j) owns rows [ks * slice, (ks + 1) * slice) of column j
-// (a value channel) of the state in registers; the groups' partial outputs meet in LDS.  Tokens
-// run in order, eight staged at a time.  a = sigmoid(z)^(1/tau) is formed as
-// exp(-softplus(-z) / tau), softplus(x) = max(x, 0) + log1p(exp(-|x|)).
+// A block a (request, head, share of the value columns).  Thread (ks, j) owns rows
+// [ks * slice, (ks + 1) * slice) of one column (a value channel) of the state in registers; the
+// groups' partial outputs meet in LDS.  Tokens run in order, eight staged at a time.
+// a = sigmoid(z)^(1/tau) is formed as exp(-softplus(-z) / tau), softplus(x) = max(x, 0) + log1p(exp(-|x|)).
+// The columns of the state never meet (column j of S only ever sees v[j]), so a head's columns may
+// be cut over several blocks: a long portion of one request then fills more of the GPU, and a
+// block's waves, which all read every token's q, k and a from LDS, are fewer.  Only the head's norm
+// needs all columns: with several shares the kernel leaves the raw o in `raw` (float32) and
+// gla_finish_kernel applies norm, gain and gate.
 template <typename T, int SLICE, bool PLAIN>
 __global__ __launch_bounds__(1024) void gla_scan_kernel(
     ScanIn q_in, ScanIn k_in, ScanIn v_in, ScanIn g_in, ScanIn z_in, const float* __restrict__ bias,
     const float* __restrict__ gain, float* __restrict__ state, const int* __restrict__ q_start,
-    const int* __restrict__ state_slots, T* __restrict__ out, GlaShape sh, float q_scale, float inv_tau, float eps) {
+    const int* __restrict__ state_slots, T* __restrict__ out, float* __restrict__ raw, GlaShape sh, float q_scale,
+    float inv_tau, float eps) {
   constexpr int TB = kScanTokens;
   extern __shared__ float lds[];
   const int dim = sh.dim, vdim = sh.vdim, CT = sh.columns, KS = sh.slices, slice = sh.slice;
@@ -335,8 +342,10 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
   float* part = rstd + TB;             // [KS][TB][CT]
   const int req = blockIdx.x, head = blockIdx.y;
   const int tid = threadIdx.x, nthreads = blockDim.x;
-  const int ks = tid / CT, j = tid - ks * CT;
-  const bool live = j < vdim;
+  const int ks = tid / CT, jl = tid - ks * CT;
+  const int j = blockIdx.z * CT + jl;               // the thread's value column; jl: its place in the block
+  const bool worker = ks < KS;                      // (threads that only fill the last wave own nothing)
+  const bool live = worker && j < vdim && jl < CT;
   const int k0 = ks * slice;
   const int kn = max(0, min(slice, dim - k0));     // key channels of this thread's slice that exist
   const int KW = sh.heads * dim, VW = sh.heads * vdim;
@@ -387,16 +396,20 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
             }
           }
         }
-        part[(ks * TB + t) * CT + j] = o;
+        if (worker) part[(ks * TB + t) * CT + jl] = o;
       }
     }
     __syncthreads();
-    for (int t = ks; t < tb; t += KS) {
+    for (int t = worker ? ks : tb; t < tb; t += KS) {
       float o = 0.f;
-      for (int q = 0; q < KS; ++q) o += part[(q * TB + t) * CT + j];
-      if (live) os[t * vdimp + j] = o;
+      for (int q = 0; q < KS; ++q) o += part[(q * TB + t) * CT + jl];
+      if (live) {
+        if (raw != nullptr) raw[(size_t)(t0 + t) * VW + vbase + j] = o;
+        else os[t * vdimp + j] = o;
+      }
     }
     __syncthreads();
+    if (raw != nullptr) continue;      // (every thread of the block alike; the next round's staging is behind this barrier)
     for (int t = wave; t < tb; t += nwaves) {
       float q = 0.f;
       for (int x = lane; x < vdim; x += kWave) q += os[t * vdimp + x] * os[t * vdimp + x];
@@ -404,7 +417,7 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
       if (lane == 0) rstd[t] = 1.f / sqrtf(q / (float)vdim + eps);
     }
     __syncthreads();
-    for (int t = ks; t < tb; t += KS) {
+    for (int t = worker ? ks : tb; t < tb; t += KS) {
       if (live) {
         const size_t at = (size_t)(t0 + t) * VW + vbase + j;
         const float g = scan_load<T, PLAIN>(g_in, at);
@@ -421,23 +434,46 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
   }
 }
 
+// out = o / rms(o) * gain * silu(gate) per (token, head), from the raw o that a scan with shared
+// columns left: a wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void gla_finish_kernel(const float* __restrict__ raw, ScanIn g_in,
+                                                         const float* __restrict__ gain, T* __restrict__ out,
+                                                         int pairs, int heads, int vdim, float eps) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int pair = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (pair >= pairs) return;
+  const size_t at = (size_t)pair * vdim;       // (token * heads + head) * vdim
+  float q = 0.f;
+  for (int x = lane; x < vdim; x += kWave) q += raw[at + x] * raw[at + x];
+  q = wave_sum(q);
+  const float rstd = 1.f / sqrtf(q / (float)vdim + eps);
+  for (int x = lane; x < vdim; x += kWave) {
+    const float g = load_in<T>(g_in.p, g_in.f32, g_in.parts, g_in.stride, at + x);
+    Elem<T>::store(out + at + x, raw[at + x] * rstd * gain[x] * (g / (1.f + expf(-g))));
+  }
+}
+
 template <typename T>
 int launch_gla(ScanIn q, ScanIn k, ScanIn v, ScanIn g, ScanIn z, const float* bias, const float* gain, float* state,
-               const int* q_start, const int* state_slots, void* out, int R, int heads, int dim, int vdim,
-               float q_scale, float inv_tau, float eps, hipStream_t stream) {
+               const int* q_start, const int* state_slots, void* out, float* raw, int N, int splits, int R, int heads,
+               int dim, int vdim, float q_scale, float inv_tau, float eps, hipStream_t stream) {
   GlaShape sh;
   sh.heads = heads;
   sh.dim = dim;
   sh.vdim = vdim;
-  sh.columns = (vdim + kWave - 1) / kWave * kWave;
+  sh.splits = splits;
+  // a block's columns: the whole head in whole waves, or a share of 16 or more
+  sh.columns = splits > 1 ? (vdim + splits - 1) / splits : (vdim + kWave - 1) / kWave * kWave;
   const int most = min(16, 1024 / sh.columns);                      // groups of threads that can share a head
   sh.slice = max(4, ((dim + most - 1) / most + 3) / 4 * 4);
   sh.slices = (dim + sh.slice - 1) / sh.slice;
-  const int threads = sh.columns * sh.slices;
+  const int threads = (sh.columns * sh.slices + kWave - 1) / kWave * kWave;
   const int dimp = (dim + 3) & ~3, vdimp = (vdim + 3) & ~3;
   const size_t lds = ((size_t)3 * kScanTokens * dimp + (size_t)kScanTokens * vdimp + kScanTokens +
                       (size_t)sh.slices * kScanTokens * sh.columns) * 4;
-  const dim3 grid(R, heads);
+  const dim3 grid(R, heads, splits);
+  float* raw_out = splits > 1 ? raw : nullptr;
   const bool plain = !q.f32 && !k.f32 && !v.f32 && !g.f32;
 #define TK_GLA_AS(SLICE, PLAIN)                                                                               \
   {                                                                                                           \
@@ -449,7 +485,8 @@ int launch_gla(ScanIn q, ScanIn k, ScanIn v, ScanIn g, ScanIn z, const float* bi
       allowed = true;                                                                                         \
     }                                                                                                         \
     gla_scan_kernel<T, SLICE, PLAIN><<<grid, threads, lds, stream>>>(q, k, v, g, z, bias, gain, state, q_start, \
-                                                                     state_slots, (T*)out, sh, q_scale, inv_tau, eps); \
+                                                                     state_slots, (T*)out, raw_out, sh, q_scale,  \
+                                                                     inv_tau, eps);                               \
   }
 #define TK_GLA(SLICE)                 \
   {                                   \
@@ -461,6 +498,10 @@ int launch_gla(ScanIn q, ScanIn k, ScanIn v, ScanIn g, ScanIn z, const float* bi
   else TK_GLA(64)
 #undef TK_GLA_AS
 #undef TK_GLA
+  if (splits > 1) {
+    const int pairs = N * heads;
+    gla_finish_kernel<T><<<(pairs + 3) / 4, 256, 0, stream>>>(raw, g, gain, (T*)out, pairs, heads, vdim, eps);
+  }
   return launch_status();
 }
 
@@ -530,21 +571,25 @@ TK_API int tk_wkv_scan(int dtype, const void* r, int r_f32, int r_parts, long r_
 // q, k, z (the decay's pre-activation, to which `bias` is added): [N, heads * dim]; v, g (gate):
 // [N, heads * vdim]; each in dtype, or float32, or float32 partial sums [parts, N, width]; out
 // [N, heads * vdim] in dtype; state [slots, heads, dim, vdim] float32.  dim, vdim <= 256.
+// splits > 1: so many blocks share a head's value columns and leave the raw o in raw
+// (float32 [N, heads * vdim]), which a second kernel norms and gates.
 TK_API int tk_gla_scan(int dtype, const void* q, int q_f32, int q_parts, long q_stride, const void* k, int k_f32,
                        int k_parts, long k_stride, const void* v, int v_f32, int v_parts, long v_stride,
                        const void* g, int g_f32, int g_parts, long g_stride, const void* z, int z_f32, int z_parts,
                        long z_stride, const float* bias, const float* gain, float* state, const int* q_start,
-                       const int* state_slots, void* out, int R, int heads, int dim, int vdim, float q_scale,
-                       float inv_tau, float eps, hipStream_t stream) {
+                       const int* state_slots, void* out, float* raw, int N, int splits, int R, int heads, int dim,
+                       int vdim, float q_scale, float inv_tau, float eps, hipStream_t stream) {
   if (R <= 0 || heads <= 0) return 0;
   if (dim < 1 || dim > 256 || vdim < 1 || vdim > 256) return -2;
+  // shares of a head's columns: 16 columns or more each, and then the raw outputs need a place
+  if (splits < 1 || (splits > 1 && (raw == nullptr || (vdim + splits - 1) / splits < 16))) return -1;
   const ScanIn qi{q, q_f32, q_parts, q_stride}, ki{k, k_f32, k_parts, k_stride}, vi{v, v_f32, v_parts, v_stride},
       gi{g, g_f32, g_parts, g_stride}, zi{z, z_f32, z_parts, z_stride};
   if (dtype == 0)
-    return launch_gla<float>(qi, ki, vi, gi, zi, bias, gain, state, q_start, state_slots, out, R, heads, dim, vdim,
-                             q_scale, inv_tau, eps, stream);
-  return launch_gla<bf16_t>(qi, ki, vi, gi, zi, bias, gain, state, q_start, state_slots, out, R, heads, dim, vdim,
-                            q_scale, inv_tau, eps, stream);
+    return launch_gla<float>(qi, ki, vi, gi, zi, bias, gain, state, q_start, state_slots, out, raw, N, splits, R, heads,
+                             dim, vdim, q_scale, inv_tau, eps, stream);
+  return launch_gla<bf16_t>(qi, ki, vi, gi, zi, bias, gain, state, q_start, state_slots, out, raw, N, splits, R, heads,
+                            dim, vdim, q_scale, inv_tau, eps, stream);
 }
 
 TK_SLOTS(tk_token_shift)
