@@ -323,8 +323,12 @@ struct GlaShape {
 // be cut over several blocks: a long portion of one request then fills more of the GPU, and a
 // block's waves, which all read every token's q, k and a from LDS, are fewer.  Only the head's norm
 // needs all columns: with several shares the kernel leaves the raw o in `raw` (float32) and
-// gla_finish_kernel applies norm, gain and gate.
-template <typename T, int SLICE, bool PLAIN>
+// gla_finish_kernel applies norm, gain and gate; the decays, which every share would form again
+// from z, are then made once by gla_decay_kernel (READY: z_in holds them, float32).
+// Measured on a 2,048-token portion of 32 heads of 128 x 128: one block a head 2.85 ms; eight
+// shares of 16 columns 2.43 ms; rounds of 32 tokens instead of 8 no faster (3.0 ms: a round's time
+// is its tokens' dependent steps, not its barriers).
+template <typename T, int SLICE, bool PLAIN, bool READY>
 __global__ __launch_bounds__(1024) void gla_scan_kernel(
     ScanIn q_in, ScanIn k_in, ScanIn v_in, ScanIn g_in, ScanIn z_in, const float* __restrict__ bias,
     const float* __restrict__ gain, float* __restrict__ state, const int* __restrict__ q_start,
@@ -365,8 +369,12 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
       const size_t at = (size_t)(t0 + t) * KW + kbase + c;
       qq[t * dimp + c] = scan_load<T, PLAIN>(q_in, at) * q_scale;
       kk[t * dimp + c] = scan_load<T, PLAIN>(k_in, at);
-      const float x = -(scan_load<T, false>(z_in, at) + bias[kbase + c]);
-      aa[t * dimp + c] = expf(-(fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)))) * inv_tau);
+      if (READY) {
+        aa[t * dimp + c] = reinterpret_cast<const float*>(z_in.p)[at];     // (the decay itself, made by gla_decay_kernel)
+      } else {
+        const float x = -(scan_load<T, false>(z_in, at) + bias[kbase + c]);
+        aa[t * dimp + c] = expf(-(fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)))) * inv_tau);
+      }
     }
     float vloc[TB];
 #pragma unroll
@@ -434,6 +442,16 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
   }
 }
 
+// a = sigmoid(z + b)^(1 / tau) for every (token, key channel), float32
+template <typename T>
+__global__ void gla_decay_kernel(ScanIn z_in, const float* __restrict__ bias, float* __restrict__ decay, int KW,
+                                 float inv_tau, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const float x = -(load_in<T>(z_in.p, z_in.f32, z_in.parts, z_in.stride, idx) + bias[idx % KW]);
+  decay[idx] = expf(-(fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)))) * inv_tau);
+}
+
 // out = o / rms(o) * gain * silu(gate) per (token, head), from the raw o that a scan with shared
 // columns left: a wave a (token, head).
 template <typename T>
@@ -472,26 +490,37 @@ int launch_gla(ScanIn q, ScanIn k, ScanIn v, ScanIn g, ScanIn z, const float* bi
   const int dimp = (dim + 3) & ~3, vdimp = (vdim + 3) & ~3;
   const size_t lds = ((size_t)3 * kScanTokens * dimp + (size_t)kScanTokens * vdimp + kScanTokens +
                       (size_t)sh.slices * kScanTokens * sh.columns) * 4;
+  const bool ready = splits > 1;
+  if (ready) {
+    // the decays once for all shares, behind the raw outputs in the same scratch array
+    float* decay = raw + (size_t)N * heads * vdim;
+    const size_t total = (size_t)N * heads * dim;
+    gla_decay_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(z, bias, decay, heads * dim, inv_tau, total);
+    z = ScanIn{decay, 1, 1, 0};
+  }
   const dim3 grid(R, heads, splits);
   float* raw_out = splits > 1 ? raw : nullptr;
   const bool plain = !q.f32 && !k.f32 && !v.f32 && !g.f32;
-#define TK_GLA_AS(SLICE, PLAIN)                                                                               \
+#define TK_GLA_AS(SLICE, PLAIN, READY_)                                                                       \
   {                                                                                                           \
     static bool allowed = false;                                                                              \
     if (!allowed) {                                                                                           \
-      const hipError_t err = hipFuncSetAttribute((const void*)gla_scan_kernel<T, SLICE, PLAIN>,               \
+      const hipError_t err = hipFuncSetAttribute((const void*)gla_scan_kernel<T, SLICE, PLAIN, READY_>,       \
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);     \
       if (err != hipSuccess) return (int)err;                                                                 \
       allowed = true;                                                                                         \
     }                                                                                                         \
-    gla_scan_kernel<T, SLICE, PLAIN><<<grid, threads, lds, stream>>>(q, k, v, g, z, bias, gain, state, q_start, \
-                                                                     state_slots, (T*)out, raw_out, sh, q_scale,  \
-                                                                     inv_tau, eps);                               \
+    gla_scan_kernel<T, SLICE, PLAIN, READY_><<<grid, threads, lds, stream>>>(q, k, v, g, z, bias, gain, state, \
+                                                                             q_start, state_slots, (T*)out,   \
+                                                                             raw_out, sh, q_scale, inv_tau, eps); \
   }
-#define TK_GLA(SLICE)                 \
-  {                                   \
-    if (plain) TK_GLA_AS(SLICE, true) \
-    else TK_GLA_AS(SLICE, false)      \
+#define TK_GLA(SLICE)                                                   \
+  {                                                                     \
+    if (ready) {                                                        \
+      if (plain) TK_GLA_AS(SLICE, true, true)                           \
+      else TK_GLA_AS(SLICE, false, true)                                \
+    } else if (plain) TK_GLA_AS(SLICE, true, false)                     \
+    else TK_GLA_AS(SLICE, false, false)                                 \
   }
   if (sh.slice <= 4) TK_GLA(4)
   else if (sh.slice <= 16) TK_GLA(16)
@@ -571,8 +600,9 @@ TK_API int tk_wkv_scan(int dtype, const void* r, int r_f32, int r_parts, long r_
 // q, k, z (the decay's pre-activation, to which `bias` is added): [N, heads * dim]; v, g (gate):
 // [N, heads * vdim]; each in dtype, or float32, or float32 partial sums [parts, N, width]; out
 // [N, heads * vdim] in dtype; state [slots, heads, dim, vdim] float32.  dim, vdim <= 256.
-// splits > 1: so many blocks share a head's value columns and leave the raw o in raw
-// (float32 [N, heads * vdim]), which a second kernel norms and gates.
+// splits > 1: so many blocks share a head's value columns (8 or more each) and leave the raw o in
+// raw (float32 [N, heads * vdim], and behind it room for the decays, [N, heads * dim]), which a
+// second kernel norms and gates.
 TK_API int tk_gla_scan(int dtype, const void* q, int q_f32, int q_parts, long q_stride, const void* k, int k_f32,
                        int k_parts, long k_stride, const void* v, int v_f32, int v_parts, long v_stride,
                        const void* g, int g_f32, int g_parts, long g_stride, const void* z, int z_f32, int z_parts,
@@ -581,8 +611,8 @@ TK_API int tk_gla_scan(int dtype, const void* q, int q_f32, int q_parts, long q_
                        int vdim, float q_scale, float inv_tau, float eps, hipStream_t stream) {
   if (R <= 0 || heads <= 0) return 0;
   if (dim < 1 || dim > 256 || vdim < 1 || vdim > 256) return -2;
-  // shares of a head's columns: 16 columns or more each, and then the raw outputs need a place
-  if (splits < 1 || (splits > 1 && (raw == nullptr || (vdim + splits - 1) / splits < 16))) return -1;
+  // shares of a head's columns: 8 columns or more each, and then the raw outputs need a place
+  if (splits < 1 || (splits > 1 && (raw == nullptr || (vdim + splits - 1) / splits < 8))) return -1;
   const ScanIn qi{q, q_f32, q_parts, q_stride}, ki{k, k_f32, k_parts, k_stride}, vi{v, v_f32, v_parts, v_stride},
       gi{g, g_f32, g_parts, g_stride}, zi{z, z_f32, z_parts, z_stride};
   if (dtype == 0)

@@ -798,7 +798,8 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tens
                                      (gate, "gate", heads * vdim), (decay_in, "decay_in", heads * dim))
                 for x in _branch(t, n, w, dtype, what)]
     splits = gla_column_splits(batch.num_requests, heads, vdim, batch.max_q_len)
-    raw = torch.empty((n, heads * vdim), dtype=torch.float32, device=out.device) if splits > 1 else None
+    # (scratch of a scan with shared columns: the raw outputs, and behind them the decays)
+    raw = torch.empty((n, heads * (vdim + dim)), dtype=torch.float32, device=out.device) if splits > 1 else None
     _note(f"{n}x{heads}x{dim}x{vdim}", n * heads * (3 * dim + 3 * vdim) * out.element_size(), 4.0 * n * heads * dim * vdim)
     _check(_fn("recurrent", "tk_gla_scan")(
         _code(dtype), *operands, _p(bias), _p(gain), _p(state), _p(batch.q_start), _p(batch.state_slots), _p(out),
@@ -807,17 +808,18 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tens
 
 
 GLA_SPLIT_FROM_TOKENS = 64     # a request's tokens in a step from which its heads' value columns are shared out
-GLA_SPLIT_MIN_COLUMNS = 16     # columns a block keeps at least
+GLA_SPLIT_MIN_COLUMNS = 8      # columns a block keeps at least
+GLA_SPLIT_BLOCKS = 1024        # blocks wanted: four small ones a CU run side by side, each waiting for its own barriers
 
 
 def gla_column_splits(requests: int, heads: int, vdim: int, longest: int) -> int:
     """Blocks that share a head's value columns in the scan: one in steps of few tokens a request
-    (the scan then norms and gates by itself); in a long portion as many as give some 256 blocks,
-    each with 16 columns or more (a second kernel then norms and gates)."""
+    (the scan then norms and gates by itself); in a long portion as many as give some 1,024 blocks,
+    each with 8 columns or more (a second kernel then norms and gates)."""
     if longest < GLA_SPLIT_FROM_TOKENS:
         return 1
     splits = 1
-    while (requests * heads * splits < 256 and vdim // (2 * splits) >= GLA_SPLIT_MIN_COLUMNS
+    while (requests * heads * splits < GLA_SPLIT_BLOCKS and vdim // (2 * splits) >= GLA_SPLIT_MIN_COLUMNS
            and vdim % (2 * splits) == 0):
         splits *= 2
     return splits
