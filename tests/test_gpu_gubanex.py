@@ -195,8 +195,10 @@ def test_gated_linear_attention_alone_in_portions_and_slots(dtype, heads, dim, v
                                dict(heads=8, kv_heads=2, dim=128, vdim=128, chunk=16, rot=64, base=1e5),
                                dict(heads=2, kv_heads=1, dim=64, vdim=64, chunk=None, rot=32),
                                dict(heads=2, kv_heads=1, dim=16, vdim=16, chunk=1, rot=2),
-                               dict(heads=4, kv_heads=1, dim=64, vdim=64, chunk=50, rot=64)],
-                         ids=["g2", "g3", "g1", "wide", "full", "one", "mid"])
+                               dict(heads=4, kv_heads=1, dim=64, vdim=64, chunk=50, rot=64),
+                               dict(heads=3, kv_heads=1, dim=20, vdim=36, chunk=9, rot=10),
+                               dict(heads=2, kv_heads=2, dim=6, vdim=2, chunk=14, rot=6)],
+                         ids=["g2", "g3", "g1", "wide", "full", "one", "mid", "pad", "tiny"])
 def test_chunked_attention_alone(dtype, a):
     """A portion from position zero, one that ends inside a page and inside a chunk, two tokens, then
     single tokens; the request's pages scattered; the position that starts a chunk given a key that
@@ -231,9 +233,13 @@ def test_chunked_attention_alone(dtype, a):
         near = plain.chunked_attention(h.double(), double(w), "l0.mix.", other, eps)[0].float()
         assert float((near - want).abs().max() / want.abs().max()) > 0.02
     pages = 40
-    store = SlotStore(0, page, {
-        "k": torch.full((pages, m["kv_heads"] * m["dim"] * page), float("nan"), dtype=dtype, device=DEV),
-        "v": torch.full((pages, m["kv_heads"] * m["vdim"] * page), float("nan"), dtype=dtype, device=DEV)})
+    # (what no token has written must not be read: NaN there; but sizes that do not fill the pages' pieces are
+    # padded with the zeros that the engine's pages start with)
+    padded = (part.key_size, part.value_size) != (m["dim"], m["vdim"])
+    assert padded == (a["dim"] % 8 != 0 or a["vdim"] % 16 != 0)
+    store = SlotStore(0, page, {name: torch.full((pages, array.elems_per_token * page), 0.0 if padded else float("nan"),
+                                                 dtype=dtype, device=DEV)
+                                for name, array in part.cache_request().arrays})
     table = [(7 * i + 3) % pages for i in range(-(-T // page))]
     got, at = [], 0
     for n in [37, 30, 2] + [1] * (T - 69):
@@ -283,13 +289,13 @@ def test_routed_experts_alone(dtype, width, ff, n, top):
 
 # -- whole models -------------------------------------------------------------------
 # Shapes that differ in everything: groups of 2, 1 and 3 query heads a kv head; key and value sizes
-# that differ; chunks that do not divide a page, a chunk of one, no chunks; rotation of a part, of
+# that differ, also ones that fill no 16-byte piece; chunks that do not divide a page, a chunk of one, no chunks; rotation of a part, of
 # the whole and of nothing; one expert a token, several, all; layers without a feed-forward; a loop
 # over the middle, over everything, none; two layers of one kind in a row.
 SHAPES = {
     "base": dict(cfg=model_json([gla(), attention(), gla(heads=4, dim=8, vdim=16), attention(chunk=9, rot=16)],
                                 loop=(1, 3, 2)), rank=8, page=16),
-    "odd": dict(cfg=model_json([attention(heads=3, kv_heads=3, dim=24, vdim=48, chunk=7, rot=12, scaling=(4.0, 1.0, 2.0, 16.0),
+    "odd": dict(cfg=model_json([attention(heads=3, kv_heads=3, dim=20, vdim=40, chunk=7, rot=12, scaling=(4.0, 1.0, 2.0, 16.0),
                                           mlp=experts(5, 1, 24)),
                                 attention(heads=6, kv_heads=2, dim=8, vdim=16, chunk=20, rot=8, mlp=None),
                                 gla(heads=3, dim=20, vdim=12, tau=3.0, mlp=experts(3, 3, 40))],

@@ -675,7 +675,10 @@ TK_API int tk_scaled_sum(int dtype, const void* a, int a_f32, int a_parts, long 
 // out, k and v written into the paged cache.  Keys and values may differ in size:
 // qkv: [N, nh * hd + nkv_in * hd + nkv_in * vd] (q heads, k heads, v heads); with nkv_in == 0
 // the input holds q heads only and nothing is stored.  Cache pages as above, the value page
-// with vd in place of hd: K page [nkv][hd/8][ps][8], V page [nkv][vd/16][ps/4][16][4].
+// with a size of its own: K page [nkv][hdp/8][ps][8], V page [nkv][vdp/16][ps/4][16][4], where
+// hdp >= hd and vdp >= vd are the sizes the pages and q_out are laid out for (hd rounded up to 8,
+// vd to 16): the channels behind hd are written as zeros into q_out and never written in the
+// pages (which start as zeros), so they add nothing to a score or an output.
 // One wave per (token, head), four waves a block, each with an LDS row of its own.
 // ---------------------------------------------------------------------------
 template <typename T, typename TIN>
@@ -684,8 +687,8 @@ __global__ void rope_norm_store_kernel(
     const float* __restrict__ k_weight, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ block_tables, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, int nh, int nkv_in, int nkv, int hd, int vd, int rot, int ps, int max_pages,
-    int unit, float eps, int num_pairs) {
+    T* __restrict__ v_cache, int nh, int nkv_in, int nkv, int hd, int vd, int hdp, int vdp, int rot, int ps,
+    int max_pages, int unit, float eps, int num_pairs) {
   __shared__ float vecs[kPairsPerBlock][kMaxHeadDim];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int heads = nh + 2 * nkv_in;
@@ -733,8 +736,8 @@ __global__ void rope_norm_store_kernel(
     }
   }
   if (is_q) {
-    T* dst = q_out + ((size_t)n * nh + head) * hd;
-    for (int d = lane; d < hd; d += kWave) Elem<T>::store(dst + d, vec[d]);
+    T* dst = q_out + ((size_t)n * nh + head) * hdp;
+    for (int d = lane; d < hdp; d += kWave) Elem<T>::store(dst + d, d < hd ? vec[d] : 0.f);
     return;
   }
   const int pos = positions[n];
@@ -742,12 +745,12 @@ __global__ void rope_norm_store_kernel(
   const int off = pos % ps;
   if (is_k) {
     const int kvh = head - nh;
-    T* base = k_cache + (size_t)page * ((size_t)nkv * hd * ps) + (size_t)kvh * hd * ps;
+    T* base = k_cache + (size_t)page * ((size_t)nkv * hdp * ps) + (size_t)kvh * hdp * ps;
     for (int d = lane; d < hd; d += kWave)
       Elem<T>::store(base + ((size_t)(d >> 3) * ps + off) * 8 + (d & 7), vec[d]);
   } else {
     const int kvh = head - nh - nkv_in;
-    T* base = v_cache + (size_t)page * ((size_t)nkv * vd * ps) + (size_t)kvh * vd * ps;
+    T* base = v_cache + (size_t)page * ((size_t)nkv * vdp * ps) + (size_t)kvh * vdp * ps;
     for (int d = lane; d < vd; d += kWave)
       Elem<T>::store(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3), vec[d]);
   }
@@ -758,10 +761,12 @@ TK_API int tk_rope_norm_store(int dtype, const void* qkv, int in_f32, int parts,
                               const float* q_weight, const float* k_weight, const float* cos_t,
                               const float* sin_t, const int* positions, const int* req_of_token,
                               const int* block_tables, void* q_out, void* k_cache, void* v_cache,
-                              int N, int nh, int nkv_in, int nkv, int hd, int vd, int rot, int ps,
-                              int max_pages, int unit, float eps, hipStream_t stream) {
+                              int N, int nh, int nkv_in, int nkv, int hd, int vd, int hdp, int vdp, int rot,
+                              int ps, int max_pages, int unit, float eps, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (hd > kMaxHeadDim || vd > kMaxHeadDim || hd % 8 != 0 || vd % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0) return -1;
+  if (hdp > kMaxHeadDim || vdp > kMaxHeadDim || hd < 1 || vd < 1 || hdp < hd || vdp < vd || hdp % 8 != 0 ||
+      vdp % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0)
+    return -1;
   if (nkv_in != 0 && nkv_in != nkv) return -1;
   if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
   const long pairs = (long)N * (nh + 2 * nkv_in);
@@ -771,7 +776,7 @@ TK_API int tk_rope_norm_store(int dtype, const void* qkv, int in_f32, int parts,
   rope_norm_store_kernel<T_, TIN_><<<grid, kWave * kPairsPerBlock, 0, stream>>>(                 \
       (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,         \
       req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, hd,   \
-      vd, rot, ps, max_pages, unit, eps, (int)pairs)
+      vd, hdp, vdp, rot, ps, max_pages, unit, eps, (int)pairs)
   if (dtype == 0) TK_RN(float, float);
   else if (in_f32) TK_RN(bf16_t, float);
   else TK_RN(bf16_t, bf16_t);

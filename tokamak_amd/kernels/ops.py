@@ -176,7 +176,7 @@ _SIGS = {
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
         "tk_rope_norm_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
         "tk_scale_softcap": [c_void_p, c_long, c_float, c_float, c_void_p],
         "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "tk_scaled_sum": [c_int, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float,
@@ -478,15 +478,18 @@ def rope_norm_store(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: 
                     store: bool = True) -> None:
     """Rotation of the first ``rotary_dim`` dims of every q and k head, then (``unit_norm``) each
     head divided by its root mean square over ``head_dim`` (times a weight, if given); q written to
-    q_out, k and v into pages.  Values are ``value_dim`` wide.  ``rotary_dim`` 0: no rotation."""
+    q_out, k and v into pages.  Values are ``value_dim`` wide.  ``rotary_dim`` 0: no rotation.
+    q_out and the pages are laid out for ``padded_sizes(head_dim, value_dim)``: the channels behind
+    the true sizes hold zeros."""
     _gpu(qkv, q_weight, k_weight, cos, sin, positions, req_of_token, block_tables, q_out, k_cache, v_cache)
     n = positions.numel()
     nkv_in = num_kv_heads if store else 0
     width = (num_heads + nkv_in) * head_dim + nkv_in * value_dim
     in_f32, parts, stride = _partials(qkv, n, width, q_out.dtype, "qkv")
-    _need(q_out.numel() >= n * num_heads * head_dim, "q_out too small")
-    _need(head_dim % 8 == 0 and value_dim % 16 == 0 and max(head_dim, value_dim) <= 512 and page_size % 8 == 0,
-          "head_dim must be a multiple of 8, value_dim of 16 (at most 512), page_size of 8")
+    hdp, vdp = padded_sizes(head_dim, value_dim)
+    _need(q_out.numel() >= n * num_heads * hdp, "q_out too small")
+    _need(min(head_dim, value_dim) >= 1 and max(hdp, vdp) <= 512 and page_size % 8 == 0,
+          "head sizes are 1 to 512, page_size a multiple of 8")
     _need(rotary_dim % 2 == 0 and rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
     _need(rotary_dim == 0 or (cos is not None and sin is not None and cos.dtype == torch.float32
                                and sin.dtype == torch.float32 and cos.numel() >= n * (rotary_dim // 2)
@@ -499,15 +502,21 @@ def rope_norm_store(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: 
     if store:
         _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_out.dtype
               and v_cache.dtype == q_out.dtype, "cache dtype must match activations")
-        _need(k_cache.numel() % (num_kv_heads * head_dim * page_size) == 0
-              and v_cache.numel() % (num_kv_heads * value_dim * page_size) == 0
-              and k_cache.numel() // head_dim == v_cache.numel() // value_dim, "cache size is not whole pages")
+        _need(k_cache.numel() % (num_kv_heads * hdp * page_size) == 0
+              and v_cache.numel() % (num_kv_heads * vdp * page_size) == 0
+              and k_cache.numel() // hdp == v_cache.numel() // vdp, "cache size is not whole pages")
     _note(f"{n}x{width}", n * width * (qkv.element_size() * parts + q_out.element_size()))
     _check(_fn("elementwise", "tk_rope_norm_store")(
         _code(q_out.dtype), _p(qkv), in_f32, parts, stride, _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
         _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
-        nkv_in, num_kv_heads, head_dim, value_dim, rotary_dim, page_size, block_tables.shape[1], int(bool(unit_norm)),
-        float(eps), _stream()), "rope_norm_store")
+        nkv_in, num_kv_heads, head_dim, value_dim, hdp, vdp, rotary_dim, page_size, block_tables.shape[1],
+        int(bool(unit_norm)), float(eps), _stream()), "rope_norm_store")
+
+
+def padded_sizes(head_dim: int, value_dim: int) -> tuple[int, int]:
+    """The sizes that cache pages are laid out for: keys in pieces of 8 channels, values in
+    blocks of 16."""
+    return -(-head_dim // 8) * 8, -(-value_dim // 16) * 16
 
 
 def scale_softcap(logits: torch.Tensor, scale: float, cap: float | None) -> None:

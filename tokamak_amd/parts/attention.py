@@ -140,12 +140,15 @@ class RotatedUnitAttention(Mixer):
         super().__init__(dtype=dtype, device=device)
         if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"num_heads ({num_heads}) must be a multiple of num_kv_heads ({num_kv_heads})")
-        if head_dim % 8 or value_dim % 16 or max(head_dim, value_dim) > 512:
-            raise ValueError(f"head_dim must be a multiple of 8 and value_dim of 16, at most 512; got {head_dim}, {value_dim}")
+        if min(head_dim, value_dim) < 1 or max(ops.padded_sizes(head_dim, value_dim)) > 512:
+            raise ValueError(f"head_dim and value_dim must be 1 to 512; got {head_dim}, {value_dim}")
         if chunk is not None and chunk < 1:
             raise ValueError(f"chunk must be >= 1, got {chunk}")
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.head_dim, self.value_dim = int(head_dim), int(value_dim)
+        # cache pages, queries and attention outputs are laid out for keys in pieces of 8 channels and
+        # values in blocks of 16: sizes that do not fill them are padded with zeros, which add nothing
+        self.key_size, self.value_size = ops.padded_sizes(self.head_dim, self.value_dim)
         self.softmax_scale = float(softmax_scale)
         self.norm_eps = None if norm_eps is None else float(norm_eps)
         self.chunk = None if chunk is None else int(chunk)
@@ -163,9 +166,14 @@ class RotatedUnitAttention(Mixer):
         q, k, v, o = self.names
         self.qkv = torch.cat([fetch(prefix + n) for n in (q, k, v)], dim=0).contiguous()
         self.o = fetch(prefix + o)
+        if self.value_size != self.value_dim:
+            # (the attention's output has the padded value size: columns of zeros in between)
+            wide = torch.zeros((self.hidden_size, self.num_heads, self.value_size), dtype=self.o.dtype, device=self.o.device)
+            wide[:, :, :self.value_dim] = self.o.view(self.hidden_size, self.num_heads, self.value_dim)
+            self.o = wide.view(self.hidden_size, self.num_heads * self.value_size).contiguous()
 
     def cache_request(self) -> CacheRequest:
-        return CacheRequest.of(window=None, k=self.num_kv_heads * self.head_dim, v=self.num_kv_heads * self.value_dim)
+        return CacheRequest.of(window=None, k=self.num_kv_heads * self.key_size, v=self.num_kv_heads * self.value_size)
 
     def step_planner(self):
         return ATTENTION_WORK
@@ -191,14 +199,14 @@ class RotatedUnitAttention(Mixer):
                 raise ops.KernelError("this attention part has no kernel for a bias on the scores")
             cos, sin, rotary_dim = position.cos, position.sin, position.rotary_dim
         tables = batch.block_tables[store.group]
-        q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
+        q = torch.empty((n, nh * self.key_size), dtype=h.dtype, device=h.device)
         ops.rope_norm_store(
             qkv, None, None, cos, sin, batch.positions, batch.req_of_token, tables, q, store.arrays["k"],
             store.arrays["v"], num_heads=nh, num_kv_heads=nkv, head_dim=hd, value_dim=vd, rotary_dim=rotary_dim,
             page_size=store.page_size, unit_norm=self.norm_eps is not None, eps=self.norm_eps or 0.0, store=writes_cache)
-        attended = torch.empty((n, nh * vd), dtype=h.dtype, device=h.device)
+        attended = torch.empty((n, nh * self.value_size), dtype=h.dtype, device=h.device)
         paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended, num_heads=nh,
-                        num_kv_heads=nkv, head_dim=hd, value_dim=vd, page_size=store.page_size,
+                        num_kv_heads=nkv, head_dim=self.key_size, value_dim=self.value_size, page_size=store.page_size,
                         scale=self.softmax_scale, chunk=self.chunk)
         return linear(attended, self.o, allow_partials=True)
 
