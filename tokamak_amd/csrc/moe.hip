@@ -235,6 +235,24 @@ union Frag8 {
 };
 
 constexpr int kTilePairs = 64;      // pairs of one expert a block takes
+constexpr int kXcds = 8;            // dies of the GPU, each with an L2 of its own; blocks go to them in turn
+
+// Which (tile, block of channels) a block of the one-dimensional grid takes.  Blocks are handed to
+// the eight dies in turn, each die has an L2 of its own, and the tiles of one expert, which read
+// the same weights, are neighbours in the tile list: so die d takes the d-th eighth of the work in
+// order, tile fastest, and the tiles of an expert at one block of channels run on one die at about
+// the same time and share the weights in its L2 (in plain grid order they land on different dies
+// and every tile streams its expert's weights from memory again).  Measured (2,048 tokens over 16
+// experts of the 8B shape, first product): plain order 0.34 PFLOP/s, this 0.41; groups of four
+// tiles by all blocks of channels per die (so that a group's activations stay in L2 as well) 0.36.
+__device__ __forceinline__ void tile_of_block(int tiles, int channel_blocks, int& tile, int& channels) {
+  const int linear = blockIdx.x;
+  const int per_die = gridDim.x / kXcds;                 // (tk_moe_grouped makes the grid a multiple of eight)
+  const int work = (linear % kXcds) * per_die + linear / kXcds;
+  tile = work < tiles * channel_blocks ? work % tiles : -1;
+  channels = work / tiles;
+}
+
 constexpr int kSortThreads = 1024;
 
 // One block: counts the pairs of every expert, lists the pairs expert by expert (order), and cuts
@@ -285,13 +303,15 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ weights, const int* __restrict__ order,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_start, const int* __restrict__ tile_count,
     const int* __restrict__ num_tiles, const float* __restrict__ pair_weight, void* __restrict__ out,
-    int N, int top, int R, int K) {
-  if ((int)blockIdx.x >= *num_tiles) return;
+    int N, int top, int R, int K, int max_tiles, int channel_blocks) {
+  int tile, channels;
+  tile_of_block(max_tiles, channel_blocks, tile, channels);
+  if (tile < 0 || tile >= *num_tiles) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kb = lane >> 4;
-  const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x], cnt = tile_count[blockIdx.x];
+  const int e = tile_expert[tile], start = tile_start[tile], cnt = tile_count[tile];
   constexpr int NT = GATED ? 2 : 4;             // tiles of 16 output channels a wave
-  const int c0 = (blockIdx.y * 4 + wave) * (16 * NT);
+  const int c0 = (channels * 4 + wave) * (16 * NT);
   if (c0 >= R) return;
   constexpr int WT = GATED ? 2 * NT : NT;       // weight fragments a step: gate and up, or down
   const bf16_t* base = weights + (size_t)e * (GATED ? 2 : 1) * R * K;
@@ -398,8 +418,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ weights, const int* __restrict__ order,
     const int* __restrict__ tile_expert, const int* __restrict__ tile_start, const int* __restrict__ tile_count,
     const int* __restrict__ num_tiles, const float* __restrict__ pair_weight, void* __restrict__ out,
-    int N, int top, int R, int K) {
-  if ((int)blockIdx.x >= *num_tiles) return;
+    int N, int top, int R, int K, int max_tiles, int channel_blocks) {
+  int tile, channels;
+  tile_of_block(max_tiles, channel_blocks, tile, channels);
+  if (tile < 0 || tile >= *num_tiles) return;
   __shared__ __attribute__((aligned(16))) bf16_t xs[ROWS * kWideLd];
   constexpr int MT = ROWS / 16;
   constexpr int XP = ROWS * 8 / 256;       // 16-byte pieces of a chunk that a thread copies
@@ -407,8 +429,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
   constexpr int WT = 4;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
-  const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x], cnt = tile_count[blockIdx.x];
-  const int c0 = (blockIdx.y * 4 + wave) * (16 * NT);
+  const int e = tile_expert[tile], start = tile_start[tile], cnt = tile_count[tile];
+  const int c0 = (channels * 4 + wave) * (16 * NT);
   const bool active = c0 < R;          // (a wave past the last channel still copies its share of the activations)
   const bf16_t* base = weights + (size_t)e * (GATED ? 2 : 1) * R * K;
   const bf16_t* wp[WT];
@@ -609,14 +631,17 @@ TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const i
   if (N <= 0 || max_tiles <= 0) return 0;
   if (K % 8 != 0 || K < 8 || R < 1 || (uintptr_t)x % 16 != 0 || (uintptr_t)weights % 16 != 0) return -1;
   const int channels = gated ? 128 : 256;      // a block's
-  const dim3 grid(max_tiles, (R + channels - 1) / channels);
+  const int channel_blocks = (R + channels - 1) / channels;
+  const int total_blocks = max_tiles * channel_blocks;
+  const dim3 grid((total_blocks + kXcds - 1) / kXcds * kXcds);      // (see tile_of_block)
   if (tile_pairs != kTilePairs) return -1;
   if (K % kWideK == 0 && rows_hint > 32) {
     // whole chunks of 64 k: the tile's activations through LDS, the next chunk asked for ahead
 #define TK_WIDE(GATED_, ROWS_)                                                                                     \
   moe_grouped_wide_kernel<GATED_, ROWS_><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order, \
                                                                    tile_expert, tile_start, tile_count, num_tiles, \
-                                                                   pair_weight, out, N, top, R, K)
+                                                                   pair_weight, out, N, top, R, K, max_tiles,      \
+                                                                   channel_blocks)
     if (gated) TK_WIDE(true, 64);
     else TK_WIDE(false, 64);
 #undef TK_WIDE
@@ -627,11 +652,13 @@ TK_API int tk_moe_grouped(int gated, const void* x, const void* weights, const i
     if (gated)                                                                                                    \
       moe_grouped_kernel<MT_, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order,    \
                                                               tile_expert, tile_start, tile_count, num_tiles,     \
-                                                              pair_weight, out, N, top, R, K);                    \
+                                                              pair_weight, out, N, top, R, K, max_tiles,          \
+                                                              channel_blocks);                                    \
     else                                                                                                          \
       moe_grouped_kernel<MT_, false><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)weights, order,   \
                                                                tile_expert, tile_start, tile_count, num_tiles,    \
-                                                               pair_weight, out, N, top, R, K);                   \
+                                                               pair_weight, out, N, top, R, K, max_tiles,         \
+                                                               channel_blocks);                                   \
   }
   // rows_hint: the most pairs an expert can have (the step's pairs): tiles are never fuller than that
   if (rows_hint <= 16) TK_GROUPED(1)
